@@ -7,7 +7,8 @@ group keys to indexes, and turns error codes into exceptions.
 
 Layers with the same need share a *group*: one pool of page ids and one block
 table per request (a page id indexes a slab of every layer of the group).  A
-group is either "all keys" (window None) or "the last W keys".  The reference
+group is either "all keys" (window None), "the last W keys", or "the keys of
+the current chunk of C positions" (window ("chunk", C)).  The reference
 keeps one identical store per layer and never evicts (ferrox-core/src/cache.rs:331-488,
 ferrox-models/src/decoder.rs:2217-2223); here a windowed group gives a page back as
 soon as every position in it is older than the window of any later query.
@@ -66,6 +67,20 @@ def _native():
     return _lib
 
 
+def _window_code(window) -> int:
+    """How a group's pages age, as the native manager numbers it: None keeps every position (-1), an int W keeps the
+    last W, ("chunk", C) keeps the positions of the chunk of C that the sequence's end lies in (-(C + 1))."""
+    if window is None:
+        return -1
+    if isinstance(window, tuple):
+        if len(window) != 2 or window[0] != "chunk" or int(window[1]) < 1:
+            raise ValueError(f"a group's window is None, a number of positions or ('chunk', size), not {window!r}")
+        return -(int(window[1]) + 1)
+    if int(window) < 0:
+        raise ValueError(f"a window of {window} positions")
+    return int(window)
+
+
 class _Core:
     """Owns one native manager."""
 
@@ -77,7 +92,7 @@ class _Core:
             raise ValueError("block_size must be >= 1")
         self.lib = _native()
         n = len(windows)
-        w = (ctypes.c_int * max(n, 1))(*[-1 if x is None else int(x) for x in windows])
+        w = (ctypes.c_int * max(n, 1))(*[_window_code(x) for x in windows])
         p = (ctypes.c_int * max(n, 1))(*[int(x) for x in num_pages])
         self.h = self.lib.fxc_create(n, w, p, block_size, n_slots)
         if not self.h:

@@ -3,7 +3,10 @@
 // Every kernel reads keys from pages [page][kv_head][slot][head_dim] and values
 // from transposed pages [page][kv_head][head_dim][slot], through a block table
 // [n_seqs, max_blocks].  A query at position p sees key t iff t <= p and, with a
-// window W > 0, p - t < W (ferrox-core/src/attention.rs:441-447, 498-513).  Head
+// window W > 0, p - t < W (ferrox-core/src/attention.rs:441-447, 498-513), or, with a
+// chunked mask of C > 0 positions, t >= floor(p / C) * C (chunks count from position 0
+// of the sequence).  A value head may have another size (vd) than a query and key
+// head (hd); the bfloat16 MFMA kernels take equal sizes, the others both.  Head
 // h reads kv head h / (n_heads / n_kv_heads) (attention.rs:432-438).  Scores,
 // softmax and the output sum are float32, in the one-pass form of
 // attention.rs:146-175 over tiles of 64 keys that start at multiples of 64, so a
@@ -31,6 +34,8 @@ struct AttnArgs {
     const int* item_tok;   // per work item: first token
     const int* item_n;     // per work item: number of queries (prefill tiles only)
     int nh, nkv, hd, bs, window;
+    int vd;              // size of a value head (and of an output head)
+    int mask_chunk;      // > 0: the chunked mask
     int bs_shift;        // log2(bs) if bs is a power of two, else -1
     int n_items;
     float scale;
@@ -46,6 +51,14 @@ static inline int log2_or_minus_one(int v) {
     while ((1 << s) < v) ++s;
     return s;
 }
+
+// the first key that a query at position p sees
+__device__ __forceinline__ int first_visible(const AttnArgs& a, int p) {
+    if (a.mask_chunk > 0) return p - p % a.mask_chunk;
+    return a.window > 0 ? max(0, p - a.window + 1) : 0;
+}
+// whether queries see a bounded stretch of keys (a window or a chunk) rather than all before them
+__device__ __forceinline__ bool bounded_keys(const AttnArgs& a) { return a.window > 0 || a.mask_chunk > 0; }
 
 // block of the table and slot in its page of key t (a shift when the page size is a power of two)
 __device__ __forceinline__ void page_slot(const AttnArgs& a, int t, int& blk, int& slot) {
@@ -91,7 +104,7 @@ __device__ __forceinline__ const T* key_row(const AttnArgs& a, const int* bt, in
 template <typename T>
 __device__ __forceinline__ const T* value_col(const AttnArgs& a, const int* bt, int kvh, int t) {
     const int page = bt[t / a.bs];
-    return (const T*)a.v_pages + ((size_t)page * a.nkv + kvh) * a.hd * a.bs + t % a.bs;  // + d * bs
+    return (const T*)a.v_pages + ((size_t)page * a.nkv + kvh) * a.vd * a.bs + t % a.bs;  // + d * bs
 }
 
 // ---------------------------------------------------------------------------
@@ -118,7 +131,7 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < TQ; ++i) pos[i] = i < n ? a.positions[tok0 + i] : -1;
     const int pmin = a.positions[tok0], pmax = a.positions[tok0 + n - 1];
-    const int kv_begin = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
+    const int kv_begin = first_visible(a, pmin);
     const int kv_end = pmax + 1;
 
     float m[TQ], l[TQ], o[HD_MAX / 64][TQ];
@@ -148,7 +161,7 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
         float al[TQ];
 #pragma unroll
         for (int i = 0; i < TQ; ++i) {
-            const bool vis = in_range && t <= pos[i] && (a.window <= 0 || pos[i] - t < a.window);
+            const bool vis = in_range && t <= pos[i] && t >= first_visible(a, pos[i]);
             const float sv = vis ? s[i] : NEG_INF;
             const float m_new = fmaxf(m[i], wave_max(sv));
             al[i] = (m_new == NEG_INF) ? 1.f : expf(m[i] - m_new);
@@ -161,7 +174,7 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
 #pragma unroll
         for (int dd = 0; dd < HD_MAX / 64; ++dd) {
             const int d = dd * 64 + lane;
-            if (d < hd) {
+            if (d < a.vd) {
 #pragma unroll
                 for (int i = 0; i < TQ; ++i) o[dd][i] *= al[i];
                 const int jn = min(64, kv_end - kt0);
@@ -177,11 +190,11 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
 #pragma unroll
     for (int dd = 0; dd < HD_MAX / 64; ++dd) {
         const int d = dd * 64 + lane;
-        if (d < hd) {
+        if (d < a.vd) {
 #pragma unroll
             for (int i = 0; i < TQ; ++i)
                 if (i < n)
-                    from_float((T*)a.out + (size_t)(tok0 + i) * a.ldo + (size_t)h * hd + d, o[dd][i] / l[i]);
+                    from_float((T*)a.out + (size_t)(tok0 + i) * a.ldo + (size_t)h * a.vd + d, o[dd][i] / l[i]);
         }
     }
 }
@@ -201,9 +214,9 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd;
     const int p = a.positions[tok];
-    const int kv_begin = max(a.window > 0 ? max(0, p - a.window + 1) : 0, split * a.chunk);
+    const int kv_begin = max(first_visible(a, p), split * a.chunk);
     const int kv_end = min(p + 1, (split + 1) * a.chunk);
-    float* po = a.part_o + (((size_t)item * a.nh + h) * a.splits + split) * hd;
+    float* po = a.part_o + (((size_t)item * a.nh + h) * a.splits + split) * a.vd;
     float* pml = a.part_ml + (((size_t)item * a.nh + h) * a.splits + split) * 2;
     if (kv_begin >= kv_end) {
         if (lane == 0) {
@@ -236,7 +249,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
 #pragma unroll
         for (int dd = 0; dd < HD_MAX / 64; ++dd) {
             const int d = dd * 64 + lane;
-            if (d < hd) {
+            if (d < a.vd) {
                 float acc = o[dd] * al;
                 const int jn = min(64, kv_end - kt0);
                 for (int j = max(0, kv_begin - kt0); j < jn; ++j)
@@ -249,7 +262,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
 #pragma unroll
     for (int dd = 0; dd < HD_MAX / 64; ++dd) {
         const int d = dd * 64 + lane;
-        if (d < hd) po[d] = o[dd];
+        if (d < a.vd) po[d] = o[dd];
     }
     if (lane == 0) {
         pml[0] = m;
@@ -266,7 +279,7 @@ __global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a) {
     __shared__ float red[2];
     const int item = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int tok = a.item_tok[item];
-    const int hd = a.hd, S = a.splits;
+    const int hd = a.vd, S = a.splits;      // (the size of an output head)
     const float* po = a.part_o + ((size_t)item * a.nh + h) * S * hd;
     const float* pml = a.part_ml + ((size_t)item * a.nh + h) * S * 2;
     // the first chunks' outputs for this thread's first dimension leave before anything else: they need no weight
@@ -589,13 +602,13 @@ __global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd;
     const int pmin = a.positions[tok0], pmax = a.positions[tok0 + n - 1];
-    const int kv_begin = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
+    const int kv_begin = first_visible(a, pmin);
     const int kv_end = pmax + 1;
     int lo = 1, hi = 0;
     const bf16* qrow = nullptr;
     if (li < n) {
         hi = a.positions[tok0 + li];
-        lo = a.window > 0 ? max(0, hi - a.window + 1) : 0;
+        lo = first_visible(a, hi);
         qrow = (const bf16*)a.q + (size_t)(tok0 + li) * a.ldq + (size_t)h * hd;
     }
     WaveAttn<HD> w;
@@ -642,19 +655,19 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
     __shared__ int page_copy[PAGE_COPY];
     int first_blk, last_blk, unused;
     PageLookup pl;
-    if (a.window <= 0) {
+    if (!bounded_keys(a)) {
         // the page ids that the split can need, whatever the position turns out to be, are copied before the
         // position has arrived (entries past the sequence's pages are read and never used)
         page_slot(a, (split + 1) * a.chunk - 1, last_blk, unused);
         last_blk = min(last_blk, a.max_blocks - 1);
         pl = stage_pages(bt, page_copy, max(0, last_blk - PAGE_COPY + 1), last_blk);
     }
-    const int first_key = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    const int first_key = first_visible(a, p);
     const int base = first_key & ~63;
     const int chunk = (((p + 1 - base + a.splits - 1) / a.splits) + 63) & ~63;
     const int kv_begin = max(first_key, base + split * chunk);
     const int kv_end = min(p + 1, base + (split + 1) * chunk);
-    if (a.window > 0) {
+    if (bounded_keys(a)) {
         page_slot(a, min(kv_begin, p), first_blk, unused);
         page_slot(a, max(kv_end - 1, 0), last_blk, unused);
         first_blk = min(first_blk, a.max_blocks - 1);
@@ -740,7 +753,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd, bs = a.bs;
     const int pmin = a.positions[tok_first], pmax = a.positions[tok_first + n_all - 1];
-    const int kv_begin = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
+    const int kv_begin = first_visible(a, pmin);
     const int kv_end = pmax + 1;
     // this wave's 16 rows
     const int tok0 = tok_first + 16 * wave, n = min(16, n_all - 16 * wave);
@@ -748,17 +761,17 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     const bf16* qrow = nullptr;
     if (li < n) {
         hi = a.positions[tok0 + li];
-        lo = a.window > 0 ? max(0, hi - a.window + 1) : 0;
+        lo = first_visible(a, hi);
         qrow = (const bf16*)a.q + (size_t)(tok0 + li) * a.ldq + (size_t)h * hd;
     }
     int w_lo = 0x7fffffff, w_hi = -1;     // keys any row of this wave can see
     int w_lo_max = 0x7fffffff, w_hi_min = -1;   // keys every row of this wave sees: [w_lo_max, w_hi_min]
     if (n > 0) {
         w_hi = a.positions[tok0 + n - 1];
-        w_lo = a.window > 0 ? max(0, a.positions[tok0] - a.window + 1) : 0;
+        w_lo = first_visible(a, a.positions[tok0]);
         if (n == 16) {                    // a wave with idle rows masks always
             w_hi_min = a.positions[tok0];
-            w_lo_max = a.window > 0 ? max(0, w_hi - a.window + 1) : 0;
+            w_lo_max = first_visible(a, w_hi);
         }
     }
     const float c2 = a.scale * LOG2E;
@@ -936,24 +949,24 @@ __global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(Att
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int bs = a.bs;
     const int pmin = a.positions[tok_first], pmax = a.positions[tok_first + n_all - 1];
-    const int kv_begin = a.window > 0 ? max(0, pmin - a.window + 1) : 0;
+    const int kv_begin = first_visible(a, pmin);
     const int kv_end = pmax + 1;
     const int tok0 = tok_first + 16 * wave, n = min(16, n_all - 16 * wave);
     int lo = 1, hi = 0;
     const bf16* qrow = nullptr;
     if (li < n) {
         hi = a.positions[tok0 + li];
-        lo = a.window > 0 ? max(0, hi - a.window + 1) : 0;
+        lo = first_visible(a, hi);
         qrow = (const bf16*)a.q + (size_t)(tok0 + li) * a.ldq + (size_t)h * HD;
     }
     int w_lo = 0x7fffffff, w_hi = -1;
     int w_lo_max = 0x7fffffff, w_hi_min = -1;
     if (n > 0) {
         w_hi = a.positions[tok0 + n - 1];
-        w_lo = a.window > 0 ? max(0, a.positions[tok0] - a.window + 1) : 0;
+        w_lo = first_visible(a, a.positions[tok0]);
         if (n == 16) {
             w_hi_min = a.positions[tok0];
-            w_lo_max = a.window > 0 ? max(0, w_hi - a.window + 1) : 0;
+            w_lo_max = first_visible(a, w_hi);
         }
     }
     const float c2 = a.scale * LOG2E;
@@ -1109,13 +1122,15 @@ FX_API int fx_debug_set(const char* key, int value) {
     return 1;
 }
 
-static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages) {
-    return dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
+static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const void* k_pages, const void* v_pages, int vd = 0) {
+    return (vd == 0 || vd == hd) && dtype == FX_BF16 && hd % 16 == 0 && bs % 16 == 0 && hd % 8 == 0 && ldq % 8 == 0 &&
            (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16 == 0);
 }
 
 // ---------------------------------------------------------------------------
-static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int bs, int window, float scale) {
+static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int bs, int window, float scale, int vd = 0, int mask_chunk = 0) {
+    FX_REQUIRE(vd >= 0 && vd <= HD_MAX, "%s: value head size %d is outside 1..%d", who, vd, HD_MAX);
+    FX_REQUIRE(mask_chunk >= 0 && !(mask_chunk > 0 && window > 0), "%s: a window (%d) or a chunked mask (%d), not both", who, window, mask_chunk);
     // (the bfloat16 kernels take a row's maximum over the raw scores and scale it once, which is the maximum of
     // the scaled scores only under a positive scale)
     FX_REQUIRE(scale > 0.f && scale < INFINITY, "%s: the scale of the scores must be positive and finite, got %g", who, (double)scale);
@@ -1138,9 +1153,11 @@ FX_API int fx_attn_tile_queries(int dtype, int hd, int bs) { return wide_items_o
 FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void* out, long ldo,
                          const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                          const int* positions, const int* item_seq, const int* item_tok, const int* item_n,
-                         int n_items, int nh, int nkv, int hd, int bs, int window, float scale, int tile_q) {
-    if (check_common("attn_tiles", dtype, nh, nkv, hd, bs, window, scale)) return 1;
-    FX_REQUIRE(tile_q == 64 || (tile_q == 128 && wide_items_ok(dtype, hd, bs) && mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)),
+                         int n_items, int nh, int nkv, int hd, int bs, int window, float scale, int tile_q,
+                         int vd, int mask_chunk) {
+    if (vd <= 0) vd = hd;
+    if (check_common("attn_tiles", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk)) return 1;
+    FX_REQUIRE(tile_q == 64 || (tile_q == 128 && wide_items_ok(dtype, hd, bs) && mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)),
                "attn_tiles: items of %d queries (64, or 128 where fx_attn_tile_queries says so)", tile_q);
     if (n_items <= 0) return 0;
     AttnArgs a = {};
@@ -1148,6 +1165,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = item_n;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
+    a.vd = vd; a.mask_chunk = mask_chunk;
     a.bs_shift = log2_or_minus_one(bs);
     a.n_items = n_items;
     dim3 grid(n_items * 4, nh), grid_blocks(8 * ceil_div((long)n_items * nh, 8));     // a wave per 16 queries / a block per item
@@ -1158,7 +1176,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     const bool two_groups = g_groups ? g_groups == 2 : (long)n_items * nh <= fx_compute_units();
     if (dtype == FX_F32)
         attn_tile_kernel<float><<<grid, 64, 0, s>>>(a);
-    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
+    else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)) {
         if (tile_q == 128 && hd == 128 && two_groups) attn_mfma_direct_kernel<128, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
         else if (tile_q == 128 && hd == 64 && two_groups) attn_mfma_direct_kernel<64, 2, 8, 2><<<grid_blocks, 1024, 0, s>>>(a);
         else if (tile_q == 128 && hd == 128) attn_mfma_direct_kernel<128, 2, 8><<<grid_blocks, 512, 0, s>>>(a);
@@ -1184,12 +1202,14 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
                               const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                               const int* positions, const int* item_seq, const int* item_tok, int n_items,
                               int nh, int nkv, int hd, int bs, int window, float scale,
-                              float* part_o, float* part_ml, int splits, int chunk, int waves) {
+                              float* part_o, float* part_ml, int splits, int chunk, int waves, int vd = 0, int mask_chunk = 0) {
+    if (vd <= 0) vd = hd;
     AttnArgs a = {};
     a.q = q; a.ldq = ldq; a.out = out; a.ldo = ldo; a.k_pages = k_pages; a.v_pages = v_pages;
     a.block_table = block_table; a.max_blocks = max_blocks; a.positions = positions;
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = nullptr;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
+    a.vd = vd; a.mask_chunk = mask_chunk;
     a.bs_shift = log2_or_minus_one(bs);
     a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.chunk = chunk;
     dim3 grid(n_items, nh, splits), grid2(n_items, nh);
@@ -1197,7 +1217,7 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
     if (dtype == FX_F32) {
         attn_decode_kernel<float><<<grid, 64, 0, s>>>(a);
         attn_decode_merge_kernel<float><<<grid2, 128, splits * sizeof(float), s>>>(a);
-    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages)) {
+    } else if (mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)) {
         const int group = nh / nkv;
         dim3 gridm(nkv * ((group + 15) / 16), n_items, splits);
         // as many waves per block (up to 8, and no more than a split has tiles) as their results fit in LDS
@@ -1243,12 +1263,13 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
                           const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                           const int* positions, const int* item_seq, const int* item_tok, int n_items,
                           int nh, int nkv, int hd, int bs, int window, float scale,
-                          float* part_o, float* part_ml, int splits, int chunk, int waves) {
+                          float* part_o, float* part_ml, int splits, int chunk, int waves, int vd, int mask_chunk) {
     if (attn_decode_check(dtype, nh, nkv, hd, bs, window, scale, splits, chunk)) return 1;
+    if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk)) return 1;
     if (n_items <= 0) return 0;
     return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
                               item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, part_o, part_ml, splits,
-                              chunk, waves);
+                              chunk, waves, vd, mask_chunk);
 }
 
 // ---------------------------------------------------------------------------

@@ -27,7 +27,7 @@ FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC"]
 HOST_LIBRARIES = ("host_runtime",)
-KERNEL_LIBRARIES = ("elementwise", "gemm", "attention", "moe", "sampling")      # what parts of a model may name
+KERNEL_LIBRARIES = ("elementwise", "gemm", "attention", "moe", "sampling", "recurrent")      # what parts of a model may name
 # kernels for measurement only (a streaming read, a copy, a loop of MFMA products, a marker): bench.py loads them,
 # no model can ask for them; their sources lie in measure/
 MEASUREMENT_LIBRARIES = ("probe",)

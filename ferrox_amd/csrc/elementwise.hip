@@ -109,7 +109,8 @@ FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* ro
 // (per-band frequency correction, attention.rs:319-333).
 // rot = 0 rotates nothing.  v is never rotated.  Key pages hold
 // [page][kv_head][slot][head_dim]; value pages hold the transpose
-// [page][kv_head][head_dim][slot], which is what the attention kernels read.
+// [page][kv_head][value head size][slot], which is what the attention kernels read (a value head's size vd
+// may differ from head_dim, the size of a query and key head).
 // ---------------------------------------------------------------------------
 // The first T * split blocks rotate: `split` blocks share a token, each computes the angles' sines
 // and cosines once and takes its part of the heads of q (in place) and of k (into its page); few
@@ -122,7 +123,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int max_blocks, T* __restrict__ k_pages, T* __restrict__ v_pages,
     int n_tokens, int split, int nh, int nkv, int hd, int bs, int rot, int interleaved, const float* __restrict__ inv_freq, int vec8,
-    const float* __restrict__ freq_factors) {
+    const float* __restrict__ freq_factors, int vd) {
     __shared__ float cs[128], sn[128];     // rot / 2 <= 128
     const int tid = threadIdx.x;
     const int half = rot >> 1;
@@ -199,11 +200,11 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     for (int i = 1; together && i < 8; ++i) together = positions[t0 + i] == pos0 + i && token_seq[t0 + i] == seq0;
     if (together) {
         const int page = block_table[(size_t)seq0 * max_blocks + pos0 / bs];
-        T* dst = v_pages + ((size_t)page * nkv + kh) * hd * bs + pos0 % bs;
-        for (int d = tid; d < hd; d += 256) {
+        T* dst = v_pages + ((size_t)page * nkv + kh) * vd * bs + pos0 % bs;
+        for (int d = tid; d < vd; d += 256) {
             uint16_t e[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) e[i] = *(const uint16_t*)(v + (size_t)(t0 + i) * ldv + (size_t)kh * hd + d);
+            for (int i = 0; i < 8; ++i) e[i] = *(const uint16_t*)(v + (size_t)(t0 + i) * ldv + (size_t)kh * vd + d);
             uint4 o;
             o.x = e[0] | ((uint32_t)e[1] << 16);
             o.y = e[2] | ((uint32_t)e[3] << 16);
@@ -213,11 +214,11 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         }
         return;
     }
-    for (int idx = tid; idx < n * hd; idx += 256) {      // tokens of different pages: element by element
-        const int i = idx / hd, d = idx - i * hd;
+    for (int idx = tid; idx < n * vd; idx += 256) {      // tokens of different pages: element by element
+        const int i = idx / vd, d = idx - i * vd;
         const int t = t0 + i, pos = positions[t];
         const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
-        v_pages[(((size_t)page * nkv + kh) * hd + d) * bs + pos % bs] = v[(size_t)t * ldv + (size_t)kh * hd + d];
+        v_pages[(((size_t)page * nkv + kh) * vd + d) * bs + pos % bs] = v[(size_t)t * ldv + (size_t)kh * vd + d];
     }
 }
 
@@ -225,7 +226,8 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
                             const void* v, int ldv, const int* positions, const int* token_seq,
                             const int* block_table, int max_blocks, void* k_pages, void* v_pages,
                             int T, int nh, int nkv, int hd, int bs, int rot, int interleaved, const float* inv_freq,
-                            const float* freq_factors) {
+                            const float* freq_factors, int vd) {
+    if (vd <= 0) vd = hd;      // a value head of the keys' size
     FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && hd > 0 && bs > 0, "rope_kv_write: bad sizes");
     FX_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary dim %d must be even and <= head_dim %d", rot, hd);
     FX_REQUIRE(rot <= 256, "rope_kv_write: rotary dim %d is more than this kernel's 256", rot);
@@ -243,12 +245,12 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
         rope_kv_write_kernel<float><<<blocks, 256, 0, s>>>((float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
                                                            positions, token_seq, block_table, max_blocks,
                                                            (float*)k_pages, (float*)v_pages, T, split, nh, nkv, hd, bs, rot,
-                                                           interleaved, inv_freq, 0, freq_factors);
+                                                           interleaved, inv_freq, 0, freq_factors, vd);
     else if (dtype == FX_BF16)
         rope_kv_write_kernel<bf16><<<blocks, 256, 0, s>>>((bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv,
                                                           positions, token_seq, block_table, max_blocks,
                                                           (bf16*)k_pages, (bf16*)v_pages, T, split, nh, nkv, hd, bs, rot,
-                                                          interleaved, inv_freq, vec8, freq_factors);
+                                                          interleaved, inv_freq, vec8, freq_factors, vd);
     else
         return fx_fail("rope_kv_write: unknown dtype %d", dtype);
     FX_CHECK_LAUNCH("rope_kv_write");
@@ -441,6 +443,87 @@ FX_API int fx_moe_combine(void* stream, float* h, const float* y, const int* inv
     }
 #undef FX_COMBINE
     FX_CHECK_LAUNCH("moe_combine");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// h[t, :] += y[t, :] * rsqrt(mean(y[t]^2) + eps) * w: a sublayer's float32 output rows are normed before they
+// join the residual stream.  One block per row; two passes over the row (the second finds it in cache).
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rmsnorm_add_kernel(float* __restrict__ h, const float* __restrict__ y,
+                                                          const void* __restrict__ w, int w_dtype, int H, float eps) {
+    __shared__ float red[4];
+    const size_t row = (size_t)blockIdx.x * H;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += 256) {
+        const float v = y[row + c];
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_sum<4>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int c = threadIdx.x; c < H; c += 256) h[row + c] += y[row + c] * scale * load_as_float(w, w_dtype, c);
+}
+
+FX_API int fx_rmsnorm_add(void* stream, float* h, const float* y, const void* w, int w_dtype, int T, int H, float eps) {
+    FX_REQUIRE(T >= 0 && H > 0, "rmsnorm_add: bad sizes T=%d H=%d", T, H);
+    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "rmsnorm_add: unknown weight dtype %d", w_dtype);
+    if (T == 0) return 0;
+    rmsnorm_add_kernel<<<T, 256, 0, (hipStream_t)stream>>>(h, y, w, w_dtype, H, eps);
+    FX_CHECK_LAUNCH("rmsnorm_add");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The weighted sum of a token's chosen experts where some router outputs are identity experts:
+//   out[t, :] = sum_j w[t, j] * (ids[t, j] < E ? y[t*k + j, :] : x[t, :])
+// in ascending j; y is float32 [T*k, H] in pair order (rows of identity pairs are never read), x the
+// feed-forward's input rows.  With norm_w the sum is then normed and added into the stream,
+//   h[t, :] += out[t, :] * rsqrt(mean(out[t]^2) + eps) * norm_w,
+// else it is added as it is.  One block per token; `out` [T, H] keeps the sums between the two passes.
+// ---------------------------------------------------------------------------
+template <typename X>
+__global__ __launch_bounds__(256) void moe_combine_identity_kernel(float* __restrict__ h, float* __restrict__ out,
+                                                                   const float* __restrict__ y, const int* __restrict__ ids,
+                                                                   const float* __restrict__ w, const X* __restrict__ x,
+                                                                   int E, int H, int k, const void* __restrict__ norm_w,
+                                                                   int norm_dtype, float eps) {
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    const size_t row = (size_t)t * H;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < H; c += 256) {
+        float acc = 0.f;
+        const float xv = to_float(x[row + c]);
+        for (int j = 0; j < k; ++j) {
+            const int e = ids[t * k + j];
+            const float v = e < E ? y[((size_t)t * k + j) * H + c] : xv;
+            acc = fmaf(w[t * k + j], v, acc);
+        }
+        out[row + c] = acc;
+        ss = fmaf(acc, acc, ss);
+    }
+    if (!norm_w) {
+        for (int c = threadIdx.x; c < H; c += 256) h[row + c] += out[row + c];      // (each thread reads what it wrote)
+        return;
+    }
+    ss = block_sum<4>(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int c = threadIdx.x; c < H; c += 256) h[row + c] += out[row + c] * scale * load_as_float(norm_w, norm_dtype, c);
+}
+
+FX_API int fx_moe_combine_identity(void* stream, float* h, float* out, const float* y, const int* ids, const float* w,
+                                   const void* x, int x_dtype, int T, int E, int H, int k, const void* norm_w,
+                                   int norm_dtype, float eps) {
+    FX_REQUIRE(T >= 0 && H > 0 && k > 0 && E >= 0, "moe_combine_identity: bad sizes");
+    FX_REQUIRE(x_dtype == FX_F32 || x_dtype == FX_BF16, "moe_combine_identity: unknown input dtype %d", x_dtype);
+    FX_REQUIRE(!norm_w || norm_dtype == FX_F32 || norm_dtype == FX_BF16, "moe_combine_identity: unknown norm weight dtype %d", norm_dtype);
+    if (T == 0) return 0;
+    hipStream_t s = (hipStream_t)stream;
+    if (x_dtype == FX_F32)
+        moe_combine_identity_kernel<float><<<T, 256, 0, s>>>(h, out, y, ids, w, (const float*)x, E, H, k, norm_w, norm_dtype, eps);
+    else
+        moe_combine_identity_kernel<bf16><<<T, 256, 0, s>>>(h, out, y, ids, w, (const bf16*)x, E, H, k, norm_w, norm_dtype, eps);
+    FX_CHECK_LAUNCH("moe_combine_identity");
     return 0;
 }
 

@@ -64,6 +64,7 @@ struct GemmArgs {
     const float* rope_freq_factors;   // rot/2 floats or null: the angle of pair i is divided by rope_freq_factors[i]
     int stream_w;  // tiled kernel: the weights are read about once (one row tile a weight matrix): load them non-temporal
     int act;     // EPI_GATED: which activation the gate goes through (ACT_*)
+    int store_act;   // EPI_STORE: what the product goes through before it is stored (SACT_*), 0 for nothing
     int vec_ok;  // 16-byte loads are legal for A and W
     int n_col_tiles, n_row_tiles;  // tiled kernels: the grid they decode block ids with
 };
@@ -186,6 +187,20 @@ __device__ __forceinline__ float gated_c(float gate, float up) {
     else if constexpr (ACT == ACT_RELU) a = fmaxf(gate, 0.0f);
     else a = silu_f(gate);
     return a * up;
+}
+// What a stored product (EPI_STORE) may go through on its way out: the activation of a feed-forward without a gate,
+// down(act(up x)).  Uniform over the launch; SACT_NONE costs one scalar compare per element.
+//   SACT_RELU2  max(x, 0)^2
+enum { SACT_NONE = 0, SACT_RELU2 = 1, SACT_RELU = 2, SACT_SILU = 3, SACT_GELU_TANH = 4, SACT_COUNT = 5 };
+__device__ __forceinline__ float stored_f(int act, float x) {
+    if (act == SACT_NONE) return x;
+    if (act == SACT_RELU2) {
+        const float r = fmaxf(x, 0.0f);
+        return r * r;
+    }
+    if (act == SACT_RELU) return fmaxf(x, 0.0f);
+    if (act == SACT_SILU) return silu_f(x);
+    return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
 }
 // f(the activation as a compile-time constant): an epilogue calls this once around its loops, so that the choice is
 // one jump per block and not work inside the loops (left inside, the compiler works out every activation for every
@@ -371,7 +386,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(GemmArgs g) {
                     float v = acc[i][j][r];
                     if (g.bias) v += bias_v[j];
                     if (EPI == EPI_STORE) {
-                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, v);
+                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, stored_f(g.store_act, v));
                     } else if (EPI == EPI_STORE_F32) {
                         ((float*)g.C)[(size_t)m * g.ldc + n] = v;
                     } else {
@@ -635,7 +650,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_wide_kernel(GemmArgs g) {
                     float v = acc[i][j][r];
                     if (g.bias) v += bias_v[j];
                     if (EPI == EPI_STORE) {
-                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, v);
+                        from_float((bf16*)g.C + (size_t)m * g.ldc + n, stored_f(g.store_act, v));
                     } else if (EPI == EPI_STORE_F32) {
                         ((float*)g.C)[(size_t)m * g.ldc + n] = v;
                     } else {
@@ -1080,7 +1095,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_bf16_skinny_kernel(GemmArgs g
             }
             if (g.bias) o += bias_v[r];
             if (EPI == EPI_STORE) {
-                from_float((bf16*)g.C + (size_t)m * g.ldc + n, o);
+                from_float((bf16*)g.C + (size_t)m * g.ldc + n, stored_f(g.store_act, o));
             } else if (EPI == EPI_STORE_F32) {
                 ((float*)g.C)[(size_t)m * g.ldc + n] = o;
             } else {
@@ -1178,7 +1193,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmArgs g) {
                     if (g.row_scale) v *= g.row_scale[ml];
                     *out += v;
                 } else {
-                    *out = v;
+                    *out = stored_f(g.store_act, v);      // (the host sets store_act for stored products only)
                 }
             }
         }
@@ -1364,7 +1379,9 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
                    const float* row_scale, const int* a_rows, const int* c_rows, const int* expert_offsets,
                    int E, int M, int N, int K, const void* norm_w, int norm_dtype, float norm_eps,
                    const int* pair_ids, int pair_div, int n_always, int always_rows, int always_from_a, long kb_rows,
-                   const float* row_ss, int row_ss_n, int act) {
+                   const float* row_ss, int row_ss_n, int act, int store_act) {
+    FX_REQUIRE(store_act >= 0 && store_act < SACT_COUNT && (store_act == 0 || (epi == EPI_STORE && !bias)),
+               "gemm: a stored activation (%d) goes with the plain stored product without bias", store_act);
     FX_REQUIRE(dtype == FX_F32 || dtype == FX_BF16, "gemm: unknown dtype %d", dtype);
     FX_REQUIRE(epi >= EPI_STORE && epi <= EPI_GATED, "gemm: unknown epilogue %d", epi);
     FX_REQUIRE(M >= 0 && N > 0 && K > 0, "gemm: bad sizes M=%d N=%d K=%d", M, N, K);
@@ -1393,7 +1410,7 @@ FX_API int fx_gemm(void* stream, int dtype, int epi, const void* A, long lda, co
     g.A = A; g.lda = lda; g.W = W; g.w_stride = w_stride; g.up_offset = up_offset;
     g.bias = bias; g.bias_dtype = bias_dtype; g.C = C; g.ldc = ldc; g.row_scale = row_scale;
     g.a_rows = a_rows; g.c_rows = c_rows; g.expert_offsets = expert_offsets; g.E = E; g.M = M; g.N = N; g.K = K;
-    g.pair_ids = pair_ids; g.pair_div = pair_div; g.act = act;
+    g.pair_ids = pair_ids; g.pair_div = pair_div; g.act = act; g.store_act = store_act;
     g.kb_stride = kb_rows * 64;
     FX_REQUIRE(kb_rows >= 0 && (kb_rows == 0 || (dtype == FX_BF16 && K % 64 == 0 && ((uintptr_t)W % 16) == 0 && lda % 8 == 0 &&
                                                  ((uintptr_t)A % 16) == 0 && (up_offset % K) == 0)),

@@ -3,7 +3,8 @@
 // ids handed out index device slabs that the Python side owns.
 //
 // Layers with the same need share a group: one pool of page ids and one block
-// table per request.  A group keeps all keys (window < 0) or the last `window`.
+// table per request.  A group keeps all keys (window -1), the last `window`, or (window -(C + 1)) the keys of
+// the current chunk of C positions.
 // The reference keeps an identical store per layer and never evicts
 // (ferrox-core/src/cache.rs:331-488); here a windowed group gives a page back as
 // soon as every later query is past it.  Rules: a page is in exactly one place
@@ -167,8 +168,11 @@ FX_API int fxc_trim(void* h, int64_t req) {
     if (!s) return fail(m, "request %ld is not admitted", (long)req);
     int freed = 0;
     for (size_t g = 0; g < m->pools.size(); ++g) {
-        if (m->windows[g] < 0) continue;
-        const int first_needed = s->length - m->windows[g] + 1;
+        const int w = m->windows[g];
+        if (w == -1) continue;
+        // a window keeps keys t >= length - W + 1; a chunked group (coded -(C + 1)) keeps those of the chunk of C
+        // positions that position `length` lies in, since a query sees no key of an earlier chunk
+        const int first_needed = w >= 0 ? s->length - w + 1 : (s->length / (-w - 1)) * (-w - 1);
         if (first_needed <= 0) continue;
         std::vector<int>& t = s->tables[g];
         const int upto = std::min<int>(first_needed / m->block_size, (int)t.size());

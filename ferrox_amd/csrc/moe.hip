@@ -70,7 +70,10 @@ __device__ __forceinline__ void wave_argmax(float& best, int& bi) {
 // (`es`: distance between the logits of neighbouring experts, 1 for a row of a [T, E] matrix)
 __device__ __forceinline__ void select_token(const float* __restrict__ row, float* score, int t, int E, int k, int renorm,
                                              int gating, int* __restrict__ ids, float* __restrict__ weights,
-                                             float* __restrict__ gate_out, int* ids_copy, long es = 1) {
+                                             float* __restrict__ gate_out, int* ids_copy, long es = 1,
+                                             const float* __restrict__ sel_bias = nullptr) {
+    // sel_bias (E floats or null): the k experts are those with the largest score + sel_bias[e]; the weights stay
+    // the scores themselves.  (A bias that steers the choice toward idle experts without changing the mixture.)
     const int lane = threadIdx.x & 63;
     if (gate_out && lane == 0) gate_out[t] = 1.0f / (1.0f + expf(-row[E * es]));
     if (E <= 64) {
@@ -88,9 +91,25 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
             sc = 1.0f / (1.0f + expf(-x));
         }
         if (!(sc >= 0.f)) sc = 0.f;     // a NaN logit makes every score NaN: such scores count as zero, so a choice stays in range
-        if (!mine) sc = -1.f;           // below every score, like the loop's start value
         float wsum = 0.f, my_w = 0.f;
         int my_id = 0;
+        if (sel_bias) {
+            float ch = mine ? sc + sel_bias[lane] : NEG_INFINITY_F;      // what the choice is made by
+            if (mine && !(ch > NEG_INFINITY_F)) ch = -3.0e38f;             // (a NaN or -inf bias: still in range, chosen last)
+            for (int j = 0; j < k; ++j) {
+                float best = ch;
+                int bi = mine ? lane : 0x7fffffff;
+                wave_argmax(best, bi);
+                const float wj = __shfl(sc, bi, 64);
+                if (lane == j) {
+                    my_w = wj;
+                    my_id = bi;
+                }
+                if (lane == bi) ch = NEG_INFINITY_F;
+                wsum += wj;
+            }
+        } else {
+        if (!mine) sc = -1.f;           // below every score, like the loop's start value
         for (int j = 0; j < k; ++j) {
             float best = sc;
             int bi = mine ? lane : 0x7fffffff;
@@ -101,6 +120,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
             }
             if (lane == bi) sc = -2.f;  // scores are >= 0; taken out of the race
             wsum += best;
+        }
         }
         if (lane < k) {
             store_shared(ids + t * k + lane, my_id);      // (at device scope: a block of this launch may sort them)
@@ -129,17 +149,26 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
     float wsum = 0.f;
     float my_w = 0.f;  // lane j keeps the weight of selection j
     for (int j = 0; j < k; ++j) {
-        float best = -1.f;
+        float best = sel_bias ? NEG_INFINITY_F : -1.f;
         int bi = 0x7fffffff;
         for (int e = lane; e < E; e += 64) {
             float v = score[e];
             if (!(v >= 0.f) && v != -2.f) v = 0.f;   // NaN counts as zero (see above): some expert in range is always found
+            if (sel_bias) {                           // chosen by score + bias; an expert already taken is out
+                v = v == -2.f ? NEG_INFINITY_F : v + sel_bias[e];
+                if (score[e] != -2.f && !(v > NEG_INFINITY_F)) v = -3.0e38f;
+            }
             if (v > best) {  // ascending e within a lane: the first maximum is kept
                 best = v;
                 bi = e;
             }
         }
         wave_argmax(best, bi);
+        if (sel_bias) {                              // the weight is the score itself (read before lane 0 marks it taken)
+            const float sv = score[bi];
+            best = sv >= 0.f ? sv : 0.f;
+            __builtin_amdgcn_wave_barrier();
+        }
         if (lane == j) my_w = best;
         if (lane == 0) {
             store_shared(ids + t * k + j, bi);
@@ -155,17 +184,19 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
 
 __global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, long ld, long es, int T,
                                                             int E, int k, int renorm, int gating, int* __restrict__ ids,
-                                                            float* __restrict__ weights, float* __restrict__ gate_out) {
+                                                            float* __restrict__ weights, float* __restrict__ gate_out,
+                                                            const float* __restrict__ sel_bias) {
     extern __shared__ float score_all[];   // 4 x E
     const int wave = threadIdx.x >> 6;
     const int t = blockIdx.x * 4 + wave;
     if (t >= T) return;
-    select_token(logits + (size_t)t * ld, score_all + wave * E, t, E, k, renorm, gating, ids, weights, gate_out, nullptr, es);
+    select_token(logits + (size_t)t * ld, score_all + wave * E, t, E, k, renorm, gating, ids, weights, gate_out, nullptr, es,
+                 sel_bias);
 }
 
 // logits of token t and expert e stand at logits[t * ld + e * es] (either of the two may be 1)
 FX_API int fx_router_select(void* stream, const float* logits, long ld, long es, int T, int E, int k, int renorm,
-                            int gating, int* ids, float* weights, float* gate_out) {
+                            int gating, int* ids, float* weights, float* gate_out, const float* sel_bias) {
     FX_REQUIRE(T >= 0, "router: bad size T=%d", T);
     FX_REQUIRE(ld >= 1 && es >= 1, "router: bad strides %ld, %ld", ld, es);
     FX_REQUIRE(E >= 1 && E <= E_MAX, "router: %d experts, this kernel takes 1..%d", E, E_MAX);
@@ -175,7 +206,7 @@ FX_API int fx_router_select(void* stream, const float* logits, long ld, long es,
     FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
     if (T == 0) return 0;
     router_select_kernel<<<(T + 3) / 4, 256, 4 * E * sizeof(float), (hipStream_t)stream>>>(logits, ld, es, T, E, k, renorm,
-                                                                                         gating, ids, weights, gate_out);
+                                                                                         gating, ids, weights, gate_out, sel_bias);
     FX_CHECK_LAUNCH("router_select");
     return 0;
 }

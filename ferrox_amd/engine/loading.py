@@ -25,11 +25,21 @@ def parse_dtype(name) -> torch.dtype:
     return DTYPES[name]
 
 
+class TensorNames(list):
+    """The names a checkpoint holds, as `build_spec` gets them, with every tensor's shape in `shapes` (name -> tuple)
+    for the sizes that a design leaves to its tensors instead of its config.json."""
+    shapes: dict
+
+    def __init__(self, source):
+        super().__init__(source.names())
+        self.shapes = {name: tuple(source.info(name)[1]) for name in self}
+
+
 def load_model(folder: str, dtype="bfloat16", device="cuda:0") -> Model:
     """config.json chooses the model class; weights are bound by tensor name."""
     arch, cfg = config_from_folder(folder)
     ckpt = Checkpoint(folder)
-    model = Model(arch.build_spec(cfg, ckpt.names()))
+    model = Model(arch.build_spec(cfg, TensorNames(ckpt)))
     model.config = cfg
     model.load(ckpt, parse_dtype(dtype), device, where=folder)
     return model

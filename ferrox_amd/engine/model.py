@@ -33,11 +33,13 @@ class Model:
         self.blocks = []
         for ls in spec.layers:
             cls = BLOCKS.get(ls.block)
-            missing = set(cls.slots) - set(ls.parts)
-            if missing:
-                raise ValueError(f"layer {ls.prefix!r}: block '{ls.block}' needs parts {sorted(missing)}")
-            parts = {slot: reg.build(ls.parts[slot]) for slot, reg in cls.slots.items()}
-            self.blocks.append(cls(parts, {slot: ls.parts[slot].prefix for slot in cls.slots}))
+            missing = set(cls.slots) - set(ls.parts) - set(getattr(cls, "optional_slots", ()))
+            unknown = set(ls.parts) - set(cls.slots)
+            if missing or unknown:
+                raise ValueError(f"layer {ls.prefix!r}: block '{ls.block}' needs parts {sorted(missing)}"
+                                 + (f" and has no place for {sorted(unknown)}" if unknown else ""))
+            parts = {slot: reg.build(ls.parts[slot]) for slot, reg in cls.slots.items() if slot in ls.parts}
+            self.blocks.append(cls(parts, {slot: ls.parts[slot].prefix for slot in parts}))
         self.final_norm = NORMS.build(spec.final_norm)
         self.head = HEADS.build(spec.head)
         self.schedule = list(spec.schedule)

@@ -27,7 +27,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to a page)")
     ap.add_argument("--block-size", type=int, default=64, help="positions per cache page")
-    ap.add_argument("--max-seqs", type=int, default=8, help="state slots (live requests)")
+    ap.add_argument("--max-seqs", type=int, default=4, help="state slots (the most requests that are live at one time)")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
 

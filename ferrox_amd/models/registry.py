@@ -51,12 +51,17 @@ def known_architectures():
 
 
 def resolve(raw_config: dict) -> Architecture:
-    """By `architectures[0]`, else by `model_type`."""
+    """By `architectures[0]`, else by `architecture`, else by `model_type`."""
     archs = raw_config.get("architectures")
     if isinstance(archs, list) and archs:
         if archs[0] in _BY_NAME:
             return _BY_NAME[archs[0]]
         raise ConfigError(f"unsupported architecture '{archs[0]}' (known: {', '.join(known_architectures())})")
+    one = raw_config.get("architecture")          # a single name instead of the list
+    if isinstance(one, str):
+        if one in _BY_NAME:
+            return _BY_NAME[one]
+        raise ConfigError(f"unsupported architecture '{one}' (known: {', '.join(known_architectures())})")
     mt = raw_config.get("model_type")
     if mt in _BY_TYPE:
         return _BY_TYPE[mt]
@@ -75,6 +80,9 @@ def _register_builtin():
     from .qwen2_moe import build_spec
     register_architecture(Architecture(Qwen2MoeConfig.architecture, Qwen2MoeConfig.model_type,
                                        Qwen2MoeConfig, build_spec))
+    from ..config.rafilix import RafilixConfig
+    from .rafilix import build_spec as rafilix_spec
+    register_architecture(Architecture(RafilixConfig.architecture, RafilixConfig.model_type, RafilixConfig, rafilix_spec))
 
 
 _register_builtin()

@@ -19,6 +19,9 @@ FX_F32, FX_BF16 = 0, 1
 EPI_STORE, EPI_STORE_F32, EPI_RESID, EPI_GATED = 0, 1, 2, 3
 # what the gate of a gated product goes through (EPI_GATED stores activation(gate) * up); ACT_* in csrc/gemm.hip
 ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "gelu": 2, "relu": 3}
+# what a stored product (EPI_STORE) may go through on its way out, the activation of a feed-forward without a
+# gate; SACT_* in csrc/gemm.hip
+STORED_ACTIVATIONS = {None: 0, "relu2": 1, "relu": 2, "silu": 3, "gelu_tanh": 4}
 GATE_SOFTMAX, GATE_SIGMOID = 0, 1
 ROPE_NEOX, ROPE_INTERLEAVED = 0, 1
 
@@ -60,7 +63,19 @@ _sigs = {
     ("elementwise", "fx_rmsnorm"): [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float],
     ("elementwise", "fx_rope_kv_write"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
                                           c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
-                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
+                                          c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_int],
+    ("elementwise", "fx_rmsnorm_add"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float],
+    ("elementwise", "fx_moe_combine_identity"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                 c_int, c_int, c_int, c_int, c_void_p, c_int, c_float],
+    ("recurrent", "fx_short_conv"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p,
+                                     c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
+    ("recurrent", "fx_delta_prepare"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long,
+                                        c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_int, c_int, c_int, c_int],
+    ("recurrent", "fx_channel_delta"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long,
+                                        c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
+    ("recurrent", "fx_gated_head_norm"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p,
+                                          c_long, c_int, c_int, c_int, c_float],
     ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
     ("elementwise", "fx_cast"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_long],
     ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -69,20 +84,20 @@ _sigs = {
     ("elementwise", "fx_feed_tokens"): [c_void_p, c_void_p, c_void_p, c_void_p, c_int],
     ("gemm", "fx_gemm"): [c_void_p, c_int, c_int, c_void_p, c_long, c_void_p, c_long, c_long, c_void_p, c_int,
                           c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
-                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int, c_int],
+                          c_void_p, c_int, c_float, c_void_p, c_int, c_int, c_int, c_int, c_long, c_void_p, c_int, c_int, c_int],
     ("gemm", "fx_qkv_rope"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p, c_long, c_int, c_int,
                               c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int],
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int],
     ("attention", "fx_attn_tile_queries"): [c_int, c_int, c_int],
     ("attention", "fx_attn_decode"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_float,
-                                      c_void_p, c_void_p, c_int, c_int, c_int],
+                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
     ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int, c_int, c_int,
-                                  c_void_p, c_void_p, c_void_p],
+                                  c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_moe_front"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
@@ -156,7 +171,7 @@ def _freq_factors(freq_factors, rotary_dim):
 _inv_freq_tables: dict = {}
 
 
-def rotary_frequencies(device, rotary_dim: int, theta: float) -> torch.Tensor | None:
+def rotary_frequencies(device, rotary_dim: int, theta: float, frequencies: tuple | None = None) -> torch.Tensor | None:
     """float32 [rotary_dim / 2] on the device: theta^(-2i/rotary_dim), worked out in float64 on the host and
     rounded once, so that the numbers do not depend on whose `powf` made them (the reference makes them in
     float32, ferrox-core/src/attention.rs:26: the last bit is its libm's).  The kernels multiply them by the
@@ -164,19 +179,28 @@ def rotary_frequencies(device, rotary_dim: int, theta: float) -> torch.Tensor | 
     recorded steps hold their addresses."""
     if rotary_dim <= 0:
         return None
-    key = (torch.device(device), int(rotary_dim), float(theta))
+    if frequencies is not None:       # an encoding's own table (float64 numbers, rounded once here)
+        frequencies = tuple(float(f) for f in frequencies)
+        if len(frequencies) != rotary_dim // 2:
+            raise KernelError(f"a table of {len(frequencies)} frequencies for {rotary_dim // 2} pairs")
+    key = (torch.device(device), int(rotary_dim), float(theta), frequencies)
     if key not in _inv_freq_tables:
-        values = [1.0 / float(theta) ** (2.0 * i / rotary_dim) for i in range(rotary_dim // 2)]
+        values = list(frequencies) if frequencies is not None else \
+            [1.0 / float(theta) ** (2.0 * i / rotary_dim) for i in range(rotary_dim // 2)]
         _inv_freq_tables[key] = torch.tensor(values, dtype=torch.float64).to(torch.float32).to(device)
     return _inv_freq_tables[key]
 
 
 def rope_kv_write(q, k, v, positions, token_seq, block_table, k_pages, v_pages, n_heads, n_kv_heads,
-                  head_dim, block_size, rotary_dim, theta, interleaved=False, freq_factors=None) -> None:
+                  head_dim, block_size, rotary_dim, theta, interleaved=False, freq_factors=None, frequencies=None,
+                  v_dim=None) -> None:
     """Rotate q in place; rotate k and write it and v into the pages (skipped when k_pages is None).
     q, k, v are 2-D views [T, heads*head_dim] with unit inner stride.  `freq_factors` (float32
-    [rotary_dim / 2] or None): the angle of pair i is divided by freq_factors[i]."""
+    [rotary_dim / 2] or None): the angle of pair i is divided by freq_factors[i].  `frequencies` (a tuple of
+    rotary_dim / 2 numbers): the pairs' frequencies, instead of theta^(-2i/rotary_dim).  `v_dim`: size of a
+    value head where it is not head_dim (v is then [T, n_kv_heads * v_dim])."""
     T = q.shape[0]
+    v_dim = int(v_dim or head_dim)
     freq_factors = _freq_factors(freq_factors, rotary_dim)
     for t in (q, k, v):
         if t.stride(-1) != 1 or t.dtype != q.dtype:
@@ -185,14 +209,16 @@ def rope_kv_write(q, k, v, positions, token_seq, block_table, k_pages, v_pages, 
         if k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
             raise KernelError("cache pages and activations differ in dtype")
         if tuple(k_pages.shape[1:]) != (n_kv_heads, block_size, head_dim) or \
-                tuple(v_pages.shape[1:]) != (n_kv_heads, head_dim, block_size):
+                tuple(v_pages.shape[1:]) != (n_kv_heads, v_dim, block_size):
             raise KernelError(f"cache pages have shapes {tuple(k_pages.shape)}, {tuple(v_pages.shape)}; expected "
-                              f"[pages,{n_kv_heads},{block_size},{head_dim}] and [pages,{n_kv_heads},{head_dim},{block_size}]")
+                              f"[pages,{n_kv_heads},{block_size},{head_dim}] and [pages,{n_kv_heads},{v_dim},{block_size}]")
+    if q.shape[1] < n_heads * head_dim or k.shape[1] < n_kv_heads * head_dim or v.shape[1] < n_kv_heads * v_dim:
+        raise KernelError("rope_kv_write: q, k or v has fewer columns than its heads need")
     _call("elementwise", "fx_rope_kv_write", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(k), k.stride(0),
           _p(v), v.stride(0), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
           _p(_i32(block_table, "block_table")), block_table.shape[1] if block_table is not None else 0,
           _p(k_pages), _p(v_pages), T, n_heads, n_kv_heads, head_dim, block_size, rotary_dim,
-          1 if interleaved else 0, _p(rotary_frequencies(q.device, rotary_dim, theta)), _p(freq_factors))
+          1 if interleaved else 0, _p(rotary_frequencies(q.device, rotary_dim, theta, frequencies)), _p(freq_factors), v_dim)
 
 
 def residual_add(h: torch.Tensor, y: torch.Tensor) -> None:
@@ -273,7 +299,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
          n_rows: int | None = None, n_out: int | None = None, up_offset: int = 0,
          norm: tuple | None = None, pair_ids: torch.Tensor | None = None, pair_div: int = 1,
          always: tuple | None = None, w_kblocked: bool = False, row_ss: tuple | None = None,
-         activation: str = "silu") -> torch.Tensor:
+         activation: str = "silu", store_activation: str | None = None) -> torch.Tensor:
     """C[m, n] = sum_k a[m, k] * w[n, k] with an epilogue.
 
     `w` is [N, K], or [E, N, K] with `expert_offsets` [E+1] (rows sorted by expert).
@@ -294,7 +320,13 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
     in (bfloat16 weights, EPI_STORE, at most 32 rows; see `can_fuse_norm`).
     `row_ss` = (ss [M, n] float32, eps): row m of the product is scaled by rsqrt(sum(ss[m]) / K + eps)
     before the bias is added (the rows of `a` are a ScaleLater's; plain stored bfloat16 product, M <= 64).
+    `store_activation` (one of STORED_ACTIVATIONS, EPI_STORE without bias): the product goes through it before it
+    is stored, e.g. "relu2" = max(x, 0)^2.
     """
+    if store_activation not in STORED_ACTIVATIONS:
+        raise KernelError(f"gemm: stored activation '{store_activation}' is not one of {sorted(k for k in STORED_ACTIVATIONS if k)}")
+    if store_activation is not None and (epilogue != EPI_STORE or bias is not None):
+        raise KernelError("gemm: a stored activation goes with the plain stored product without bias")
     if row_ss is not None:
         ss = row_ss[0]
         if ss.dtype != torch.float32 or ss.dim() != 2 or not ss.is_contiguous() or ss.shape[0] != a.shape[0]:
@@ -362,7 +394,7 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, epilogue: int = EPI_STORE, out: to
           _p(_i32(pair_ids, "pair_ids")), int(pair_div),
           n_always, always_rows, always_from_a, n_w if w_kblocked else 0,
           _p(row_ss[0]) if row_ss is not None else None, row_ss[0].shape[1] if row_ss is not None else 0,
-          ACTIVATIONS[activation])
+          ACTIVATIONS[activation], STORED_ACTIVATIONS[store_activation])
     return out
 
 
@@ -443,14 +475,29 @@ def attention_tile_queries(dtype, head_dim: int, block_size: int) -> int:
 
 
 def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok, item_n,
-                    n_heads, n_kv_heads, head_dim, block_size, window, scale, tile_q: int = 64) -> None:
+                    n_heads, n_kv_heads, head_dim, block_size, window, scale, tile_q: int = 64, mask_chunk: int = 0,
+                    v_dim: int | None = None) -> None:
     """Blocks of queries: item i is item_n[i] <= tile_q consecutive tokens of sequence item_seq[i] from token
-    item_tok[i] on; tile_q is 64 or attention_tile_queries(...)."""
+    item_tok[i] on; tile_q is 64 or attention_tile_queries(...).  `mask_chunk` > 0: the chunked mask (a query sees
+    the keys of its own chunk of that many positions) instead of a window.  `v_dim`: size of a value head where it
+    is not head_dim; `out` is [T, n_heads * v_dim]."""
+    _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, int(v_dim or head_dim), block_size)
     _call("attention", "fx_attn_tiles", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0),
           _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")),
           _p(_i32(item_n, "item_n")), item_seq.numel(), n_heads, n_kv_heads, head_dim, block_size,
-          int(window or 0), float(scale), int(tile_q))
+          int(window or 0), float(scale), int(tile_q), int(v_dim or head_dim), int(mask_chunk or 0))
+
+
+def _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, v_dim, block_size) -> None:
+    """The kernels index by these sizes: the operands must hold them."""
+    if q.shape[1] < n_heads * head_dim or out.shape[1] < n_heads * v_dim or out.shape[0] < q.shape[0]:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} for {n_heads} heads of {head_dim} / {v_dim}")
+    if tuple(k_pages.shape[1:]) != (n_kv_heads, block_size, head_dim) or tuple(v_pages.shape[1:]) != (n_kv_heads, v_dim, block_size):
+        raise KernelError(f"attention: cache pages have shapes {tuple(k_pages.shape)}, {tuple(v_pages.shape)}; expected "
+                          f"[pages,{n_kv_heads},{block_size},{head_dim}] and [pages,{n_kv_heads},{v_dim},{block_size}]")
+    if q.dtype != out.dtype or k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
+        raise KernelError("attention: queries, output and cache pages differ in dtype")
 
 
 SPLIT_PARTIAL_ROUNDS = True      # decode attention: more chunks where the blocks' last round over the CUs would be far from full
@@ -481,31 +528,37 @@ def decode_attention_chunk(n_items: int, n_heads: int, n_kv_heads: int, max_kv_l
 
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
                      n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None,
-                     waves=0) -> None:
+                     waves=0, mask_chunk: int = 0, v_dim: int | None = None) -> None:
     """Single queries.  The keys go to ceil(max_kv_len / chunk) blocks whose results are merged in ascending
     order.  float32 cuts them at multiples of `chunk`, 256 by default (so that a result does not depend on the
     batch); bfloat16, whose blocks of up to eight waves share a chunk, cuts every sequence's own range of keys (from
     its window's first key to its position) into that many equal chunks of whole tiles of 64, `chunk` by default as
     `decode_attention_chunk` picks it.  `waves`: waves per block, 0 for the launch's own choice."""
     n = item_seq.numel()
+    v_dim = int(v_dim or head_dim)
+    _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, v_dim, block_size)
     if chunk is None:
         chunk = 256
         if q.dtype == torch.bfloat16:
             chunk = decode_attention_chunk(n, n_heads, n_kv_heads, max_kv_len, compute_units(q.device))
     splits = max(1, -(-max_kv_len // chunk))
-    part_o = torch.empty((n, n_heads, splits, head_dim), dtype=torch.float32, device=q.device)
+    part_o = torch.empty((n, n_heads, splits, v_dim), dtype=torch.float32, device=q.device)
     part_ml = torch.empty((n, n_heads, splits, 2), dtype=torch.float32, device=q.device)
     _call("attention", "fx_attn_decode", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0),
           _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")), n,
           n_heads, n_kv_heads, head_dim, block_size, int(window or 0), float(scale),
-          _p(part_o), _p(part_ml), splits, chunk, int(waves))
+          _p(part_o), _p(part_ml), splits, chunk, int(waves), v_dim, int(mask_chunk or 0))
 
 
-def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
+def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False, selection_bias=None):
     """From float32 router logits [T, >= E (+1)] (any strides, so also the transpose of an
     [E (+1), T] product): (ids int32 [T,k], weights float32 [T,k], gate float32 [T] =
-    sigmoid(logits[:, E]) or None)."""
+    sigmoid(logits[:, E]) or None).  `selection_bias` (float32 [E]): the experts are chosen by score + bias,
+    the weights are the scores."""
+    if selection_bias is not None and (selection_bias.dtype != torch.float32 or not selection_bias.is_contiguous()
+                                       or selection_bias.numel() != n_experts):
+        raise KernelError(f"router_select: the selection bias must be {n_experts} contiguous float32 values")
     if logits.dtype != torch.float32 or logits.dim() != 2 or min(logits.stride()) < 1:
         raise KernelError("router_select: logits must be a float32 [T, E] matrix")
     T = logits.shape[0]
@@ -515,7 +568,7 @@ def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gat
     if logits.shape[1] < n_experts + (1 if has_gate else 0):
         raise KernelError(f"router_select: {logits.shape[1]} columns for {n_experts} experts")
     _call("moe", "fx_router_select", _stream(), _p(logits), logits.stride(0), logits.stride(1), T, n_experts, top_k,
-          1 if renorm else 0, gating, _p(ids), _p(weights), _p(gate))
+          1 if renorm else 0, gating, _p(ids), _p(weights), _p(gate), _p(selection_bias))
     return ids, weights, gate
 
 
@@ -631,3 +684,119 @@ def sample(logits: torch.Tensor, *, temperature=None, draw=None, top_k=None, top
           _p(temperature), _p(_i32(top_k, "top_k")), _p(top_p), _p(rep_penalty), _p(presence), _p(frequency),
           _p(draw), _p(_i32(hist, "hist")), _p(_i32(hist_start, "hist_start")), _p(out))
     return out
+
+
+# ---------------------------------------------------------------------------
+# norms after a sublayer, identity experts, recurrent mixers
+# ---------------------------------------------------------------------------
+def rmsnorm_add(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float) -> None:
+    """h[t] += y[t] * rsqrt(mean(y[t]^2) + eps) * weight: float32 rows of a sublayer's output, normed as they join
+    the residual stream."""
+    if h.dtype != torch.float32 or y.dtype != torch.float32 or h.shape != y.shape or not h.is_contiguous() or not y.is_contiguous():
+        raise KernelError("rmsnorm_add wants contiguous float32 h and y of one shape")
+    T, H = h.shape
+    if weight.numel() != H or not weight.is_contiguous():
+        raise KernelError(f"rmsnorm_add: weight of {weight.numel()} elements for width {H}")
+    _call("elementwise", "fx_rmsnorm_add", _stream(), _p(h), _p(y), _p(weight), dtype_code(weight.dtype), T, H, float(eps))
+
+
+def moe_combine_identity(h, y, ids, weights, x, n_experts: int, post_norm=None) -> None:
+    """h[t] += N(sum_j weights[t, j] * (y[t*k + j] if ids[t, j] < n_experts else x[t])), N the RMS norm
+    `post_norm` = (weight, eps) or nothing.  y: float32 [T*k, H] in pair order (rows of pairs that chose an
+    identity expert, ids >= n_experts, are never read); x: the feed-forward's input rows [T, H]."""
+    T, H = h.shape
+    k = ids.shape[1]
+    if h.dtype != torch.float32 or y.dtype != torch.float32 or weights.dtype != torch.float32 or not h.is_contiguous():
+        raise KernelError("moe_combine_identity works on float32")
+    if not y.is_contiguous() or y.shape[0] < T * k or y.shape[1] != H or tuple(x.shape) != (T, H) or not x.is_contiguous():
+        raise KernelError(f"moe_combine_identity: y {tuple(y.shape)} / x {tuple(x.shape)} for {T} tokens, {k} choices, width {H}")
+    if tuple(weights.shape) != (T, k) or not weights.is_contiguous() or not ids.is_contiguous():
+        raise KernelError("moe_combine_identity: ids and weights must be contiguous [T, k]")
+    nw, eps = post_norm if post_norm is not None else (None, 0.0)
+    if nw is not None and (nw.numel() != H or not nw.is_contiguous()):
+        raise KernelError(f"moe_combine_identity: norm weight of {nw.numel()} elements for width {H}")
+    out = torch.empty((T, H), dtype=torch.float32, device=h.device)
+    _call("elementwise", "fx_moe_combine_identity", _stream(), _p(h), _p(out), _p(y), _p(_i32(ids, "ids")), _p(weights), _p(x),
+          dtype_code(x.dtype), T, int(n_experts), H, k, _p(nw), dtype_code(nw.dtype) if nw is not None else 0, float(eps))
+
+
+def _f32_rows(t, what, cols):
+    if t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or t.shape[1] < cols:
+        raise KernelError(f"{what} must be float32 rows of at least {cols} columns with unit inner stride")
+    return t
+
+
+def short_conv(x, taps, state, token_seq, seq_starts, slot_ids, n_seqs: int) -> torch.Tensor:
+    """y[t, c] = silu(sum_j taps[c, n-1-j] x[t-j, c]) over each sequence's own tokens, the n-1 inputs from before
+    the step coming from state[slot, c, :] (oldest first), which afterwards holds the step's last n-1 inputs.
+    x: float32 [T, C] rows (any row stride); taps [C, n]; state float32 [slots, C, n-1]; sequence s owns tokens
+    [seq_starts[s], seq_starts[s+1]) and slot slot_ids[s].  Returns float32 [T, C]."""
+    T, C = x.shape
+    n = taps.shape[1]
+    _f32_rows(x, "short_conv: x", C)
+    if tuple(taps.shape) != (C, n) or not taps.is_contiguous():
+        raise KernelError(f"short_conv: taps {tuple(taps.shape)} for {C} channels")
+    if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (C, max(n - 1, 0)):
+        raise KernelError(f"short_conv: state {tuple(state.shape)} for [slots, {C}, {n - 1}]")
+    if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs or token_seq.numel() < T:
+        raise KernelError("short_conv: the step's index tensors are shorter than its sequences and tokens")
+    y = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    _call("recurrent", "fx_short_conv", _stream(), _p(x), x.stride(0), _p(y), y.stride(0), _p(taps), dtype_code(taps.dtype), n,
+          _p(state), _p(_i32(token_seq, "token_seq")), _p(_i32(seq_starts, "seq_starts")), _p(_i32(slot_ids, "slot_ids")),
+          T, int(n_seqs), C)
+    return y
+
+
+def delta_prepare(q, k, a, b, A_log, dt_bias, n_heads: int, n_kv_heads: int, key_dim: int):
+    """From convolved q, k [T, G*D], the decay's projection a [T, H*D] and the step size's b [T, H] (float32 rows):
+    (q / |q| / sqrt(D), k / |k|, exp(-exp(A_log[h]) softplus(a + dt_bias)), sigmoid(b)), all float32 contiguous."""
+    T = q.shape[0]
+    H, G, D = int(n_heads), int(n_kv_heads), int(key_dim)
+    _f32_rows(q, "delta_prepare: q", G * D), _f32_rows(k, "delta_prepare: k", G * D)
+    _f32_rows(a, "delta_prepare: a", H * D), _f32_rows(b, "delta_prepare: b", H)
+    if A_log.numel() != H or dt_bias.numel() != H * D or A_log.dtype != dt_bias.dtype or not A_log.is_contiguous() \
+            or not dt_bias.is_contiguous():
+        raise KernelError(f"delta_prepare: A_log {tuple(A_log.shape)} / dt_bias {tuple(dt_bias.shape)} for {H} heads of {D}")
+    dev = q.device
+    qn = torch.empty((T, G * D), dtype=torch.float32, device=dev)
+    kn = torch.empty((T, G * D), dtype=torch.float32, device=dev)
+    decay = torch.empty((T, H * D), dtype=torch.float32, device=dev)
+    beta = torch.empty((T, H), dtype=torch.float32, device=dev)
+    _call("recurrent", "fx_delta_prepare", _stream(), _p(q), q.stride(0), _p(k), k.stride(0), _p(a), a.stride(0), _p(b),
+          b.stride(0), _p(A_log), _p(dt_bias), dtype_code(A_log.dtype), _p(qn), _p(kn), _p(decay), _p(beta), T, H, G, D)
+    return qn, kn, decay, beta
+
+
+def channel_delta(qn, kn, decay, beta, v, state, seq_starts, slot_ids, n_seqs: int, n_heads: int, n_kv_heads: int,
+                  key_dim: int, v_dim: int) -> torch.Tensor:
+    """The gated delta rule with a decay per key channel, over each sequence's tokens in order, from and into
+    state[slot] (float32 [slots, H, D, V]):  S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;
+    o_t = S^T q_t.  Returns o float32 [T, H*V]."""
+    T = qn.shape[0]
+    H, G, D, V = int(n_heads), int(n_kv_heads), int(key_dim), int(v_dim)
+    for t, cols, what in ((qn, G * D, "q"), (kn, G * D, "k"), (decay, H * D, "decay"), (beta, H, "beta")):
+        if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (T, cols):
+            raise KernelError(f"channel_delta: {what} must be contiguous float32 [{T}, {cols}]")
+    _f32_rows(v, "channel_delta: v", H * V)
+    if v.shape[0] != T or state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, D, V):
+        raise KernelError(f"channel_delta: v {tuple(v.shape)} / state {tuple(state.shape)} for [slots, {H}, {D}, {V}]")
+    if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs:
+        raise KernelError("channel_delta: the step's index tensors are shorter than its sequences")
+    out = torch.empty((T, H * V), dtype=torch.float32, device=qn.device)
+    _call("recurrent", "fx_channel_delta", _stream(), _p(qn), _p(kn), _p(decay), _p(beta), _p(v), v.stride(0), _p(out),
+          out.stride(0), _p(state), _p(_i32(seq_starts, "seq_starts")), _p(_i32(slot_ids, "slot_ids")), int(n_seqs), H, G, D, V)
+    return out
+
+
+def gated_head_norm(o, gate, weight, eps: float, n_heads: int, v_dim: int, out_dtype) -> torch.Tensor:
+    """y[t, h, :] = o[t, h, :] / rms(o[t, h, :]) * weight * sigmoid(gate[t, h, :]) in `out_dtype`; o and gate are
+    float32 rows [T, H*V], weight [V] is shared by the heads."""
+    T = o.shape[0]
+    H, V = int(n_heads), int(v_dim)
+    _f32_rows(o, "gated_head_norm: o", H * V), _f32_rows(gate, "gated_head_norm: gate", H * V)
+    if gate.shape[0] != T or weight.numel() != V or not weight.is_contiguous():
+        raise KernelError(f"gated_head_norm: gate {tuple(gate.shape)} / weight {tuple(weight.shape)} for {T} x {H} heads of {V}")
+    y = torch.empty((T, H * V), dtype=out_dtype, device=o.device)
+    _call("recurrent", "fx_gated_head_norm", _stream(), dtype_code(out_dtype), _p(o), o.stride(0), _p(gate), gate.stride(0),
+          _p(weight), dtype_code(weight.dtype), _p(y), y.stride(0), T, H, V, float(eps))
+    return y

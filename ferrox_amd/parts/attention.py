@@ -60,12 +60,22 @@ def attention_items(ctx, tile_q: int = 64):
 class PagedAttention(Mixer):
     kernel_libraries = ("elementwise", "gemm", "attention")
     graph_safe = True      # its launches depend on device data and on sizes that are fixed per graph
+    takes_post_norm = True     # forward(..., post_norm=(weight, eps)) norms the output rows before they join the stream
+    TENSORS = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+               "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
+               "q_norm": "q_norm.", "k_norm": "k_norm."}
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, bias: bool,
                  position: PartSpec, window: int | None = None, scale: float | None = None,
-                 qk_norm: PartSpec | None = None):
+                 qk_norm: PartSpec | None = None, v_dim: int | None = None, chunk: int | None = None,
+                 names: dict | None = None):
         """`qk_norm`: kind and arguments of a norm over head_dim; two of them are built, with tensors under
-        `q_norm.` and `k_norm.`, and applied to every head of q and of k before the rotation."""
+        `q_norm.` and `k_norm.`, and applied to every head of q and of k before the rotation.
+        `v_dim`: size of a value head where it differs from head_dim (the size of a query and key head).
+        `chunk`: a query at position p sees the keys t <= p of its own chunk only, floor(t / chunk) == floor(p / chunk),
+        chunks counted from position 0 of the sequence.
+        `names`: what the checkpoint calls this part's tensors, where that differs from `TENSORS` (the prefixes of
+        the two norms among them)."""
         if n_heads % n_kv_heads:
             raise ValueError(f"n_heads {n_heads} is not a multiple of n_kv_heads {n_kv_heads}")
         if head_dim % limits.HEAD_DIM_STEP or not limits.HEAD_DIM_STEP <= head_dim <= limits.HEAD_DIM_MAX:
@@ -74,41 +84,54 @@ class PagedAttention(Mixer):
         self.hidden_size, self.n_heads, self.n_kv_heads, self.head_dim = hidden_size, n_heads, n_kv_heads, head_dim
         self.bias = bool(bias)
         self.window = int(window) if window else None
+        self.chunk = int(chunk) if chunk else None
+        if self.window and self.chunk:
+            raise ValueError("an attention layer has a sliding window or a chunked mask, not both")
+        self.v_dim = int(v_dim) if v_dim else head_dim
+        if not 1 <= self.v_dim <= limits.HEAD_DIM_MAX:
+            raise ValueError(f"v_dim {self.v_dim}: the attention kernels take up to {limits.HEAD_DIM_MAX}")
+        self.names = dict(self.TENSORS, **(names or {}))
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # attention.rs:433
         if not 0.0 < self.scale < math.inf:
             raise ValueError(f"the scale of the attention scores must be positive and finite, got {self.scale}")
         self.position = POSITION_ENCODINGS.build(position)
         self._position_prefix = position.prefix or ""       # where the encoding's own tensors (if any) are named
-        self.qw, self.kvw = n_heads * head_dim, n_kv_heads * head_dim
+        self.qw, self.kvw, self.vw, self.ow = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * self.v_dim, n_heads * self.v_dim
         self.qkv = self.o_proj = None
         self.q_norm = self.k_norm = None
         if qk_norm is not None:
             self.q_norm, self.k_norm = (NORMS.build(PartSpec(qk_norm.kind, dict(qk_norm.args))) for _ in range(2))
 
     def children(self):
-        norms = [("q_norm.", self.q_norm), ("k_norm.", self.k_norm)] if self.q_norm is not None else []
+        norms = [(self.names["q_norm"], self.q_norm), (self.names["k_norm"], self.k_norm)] if self.q_norm is not None else []
         return [(self._position_prefix, self.position)] + norms
 
     def param_specs(self):
-        H = self.hidden_size
-        specs = {"q_proj.weight": ParamSpec((self.qw, H)), "k_proj.weight": ParamSpec((self.kvw, H)),
-                 "v_proj.weight": ParamSpec((self.kvw, H)), "o_proj.weight": ParamSpec((H, self.qw))}
+        H, n = self.hidden_size, self.names
+        specs = {n["q"]: ParamSpec((self.qw, H)), n["k"]: ParamSpec((self.kvw, H)),
+                 n["v"]: ParamSpec((self.vw, H)), n["o"]: ParamSpec((H, self.ow))}
         if self.bias:
-            specs.update({"q_proj.bias": ParamSpec((self.qw,)), "k_proj.bias": ParamSpec((self.kvw,)),
-                          "v_proj.bias": ParamSpec((self.kvw,))})
+            specs.update({n["q_bias"]: ParamSpec((self.qw,)), n["k_bias"]: ParamSpec((self.kvw,)),
+                          n["v_bias"]: ParamSpec((self.vw,))})
         return specs
 
     def load(self, fetch):
-        w = torch.cat(same_dtype([fetch("q_proj.weight"), fetch("k_proj.weight"), fetch("v_proj.weight")]), dim=0)
+        n = self.names
+        w = torch.cat(same_dtype([fetch(n["q"]), fetch(n["k"]), fetch(n["v"])]), dim=0)
         b = None
         if self.bias:
-            b = torch.cat(same_dtype([fetch("q_proj.bias"), fetch("k_proj.bias"), fetch("v_proj.bias")]), dim=0)
+            b = torch.cat(same_dtype([fetch(n["q_bias"]), fetch(n["k_bias"]), fetch(n["v_bias"])]), dim=0)
         self.qkv = Linear(w, b)
-        self.o_proj = Linear(fetch("o_proj.weight"))
+        self.o_proj = Linear(fetch(n["o"]))
 
     def page_shapes(self, block_size: int) -> dict:
         return {"k": (self.n_kv_heads, block_size, self.head_dim),
-                "v": (self.n_kv_heads, self.head_dim, block_size)}
+                "v": (self.n_kv_heads, self.v_dim, block_size)}
+
+    def cache_group(self):
+        if self.chunk:      # pages age with the chunks: those of a chunk that has ended are given back
+            return ("chunk", self.chunk), ("chunk", self.chunk)
+        return super().cache_group()
 
     def forward_from_residual(self, norm, ctx, cache, residual) -> bool:
         """Few tokens: the norm is applied inside the q/k/v product (up to 16 rows it saves a launch; with
@@ -136,7 +159,7 @@ class PagedAttention(Mixer):
         portion deep in a prompt: 603 against 784 us at 16 heads); else items of 128 if they still number about
         one evenly loaded block per CU (blocks of a portion that starts a prompt differ in work up to the portion's
         length in keys and count by their mean share of the longest; +8-26 % from 448 such blocks on); else 64."""
-        if ctx.recorded:
+        if ctx.recorded or self.v_dim != self.head_dim:      # (the kernels for unequal head sizes take items of 64)
             return 64
         widest = ops.attention_tile_queries(dtype, self.head_dim, block_size)
         if widest == 64:
@@ -177,12 +200,13 @@ class PagedAttention(Mixer):
         k = self.k_norm.forward(heads, ctx, rows=k_rows).view(T, self.kvw)
         return q, k, v
 
-    def forward(self, x, ctx, cache, residual, qkv=None) -> None:
+    def forward(self, x, ctx, cache, residual, qkv=None, post_norm=None) -> None:
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
         rot = self.position.rotary()
         debug.region("qkv")
-        fused = (qkv is None and self.q_norm is None and rot is not None
+        fused = (qkv is None and self.q_norm is None and rot is not None and rot.frequencies is None
+                 and self.v_dim == self.head_dim
                  and ops.can_qkv_rope(x, self.qkv.weight, ctx.n_tokens, self.head_dim, rot.rotary_dim, rot.interleaved))
         if fused:
             # few tokens: rotation and cache write happen in the product's epilogue
@@ -209,18 +233,22 @@ class PagedAttention(Mixer):
             ops.rope_kv_write(q, k, v, ctx.positions, ctx.token_seq, table,
                               k_pages if cache.writes else None, v_pages if cache.writes else None,
                               self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot.rotary_dim, rot.theta,
-                              rot.interleaved, rot.freq_factors)
+                              rot.interleaved, rot.freq_factors, frequencies=rot.frequencies, v_dim=self.v_dim)
         debug.region("attention")
-        out = torch.empty((ctx.n_tokens, self.qw), dtype=qkv.dtype, device=qkv.device)
-        tile_q = ctx.memo(f"attention tile {self.n_heads} {self.head_dim} {cache.block_size} {q.dtype}",
+        out = torch.empty((ctx.n_tokens, self.ow), dtype=qkv.dtype, device=qkv.device)
+        tile_q = ctx.memo(f"attention tile {self.n_heads} {self.head_dim} {self.v_dim} {cache.block_size} {q.dtype}",
                           lambda: self.tile_queries(ctx, q.dtype, cache.block_size))
         items = ctx.memo(f"attention_items {tile_q}", lambda: attention_items(ctx, tile_q))
         common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)
+        mask = dict(mask_chunk=self.chunk or 0, v_dim=self.v_dim)
         if items["n_tiles"]:
             ops.attention_tiles(q, out, k_pages, v_pages, table, ctx.positions,
-                                items["tile_seq"], items["tile_tok"], items["tile_n"], *common, tile_q=tile_q)
+                                items["tile_seq"], items["tile_tok"], items["tile_n"], *common, tile_q=tile_q, **mask)
         if items["n_decode"]:
             ops.attention_decode(q, out, k_pages, v_pages, table, ctx.positions,
-                                 items["dec_seq"], items["dec_tok"], *common, max_kv_len=items["max_kv"])
+                                 items["dec_seq"], items["dec_tok"], *common, max_kv_len=items["max_kv"], **mask)
         debug.region("o_proj")
-        self.o_proj(out, epilogue=ops.EPI_RESID, out=residual)
+        if post_norm is None:
+            self.o_proj(out, epilogue=ops.EPI_RESID, out=residual)
+        else:       # the output rows are normed before they join the stream: float32 rows, then one kernel norms and adds
+            ops.rmsnorm_add(residual, self.o_proj(out, epilogue=ops.EPI_STORE_F32), post_norm[0], post_norm[1])

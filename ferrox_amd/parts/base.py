@@ -229,11 +229,14 @@ class Rotary:
     """A rotation that the kernels apply themselves while they write the cache: pair i of the first
     `rotary_dim` dimensions of every q and k head turns by pos * theta^(-2i/rotary_dim), divided by
     freq_factors[i] if a table is given (float32 [rotary_dim / 2] on the device).  Pairs are
-    (i, i + rotary_dim/2), or (2i, 2i+1) when `interleaved`.  rotary_dim 0 rotates nothing."""
+    (i, i + rotary_dim/2), or (2i, 2i+1) when `interleaved`.  rotary_dim 0 rotates nothing.
+    `frequencies` (a tuple of rotary_dim / 2 numbers) replaces theta^(-2i/rotary_dim) by a table of the
+    encoding's own: pair i turns by pos * frequencies[i], the product taken in float32."""
     rotary_dim: int
     theta: float
     interleaved: bool = False
     freq_factors: torch.Tensor | None = None
+    frequencies: tuple | None = None
 
 
 class PositionEncoding(Part):

@@ -1,6 +1,8 @@
 """Arrangements of a mixer, a feed-forward and norms in one layer."""
 from __future__ import annotations
 
+import torch
+
 from .. import debug
 from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block
 
@@ -45,3 +47,50 @@ class PreNormBlock(Block):
             self.ffn.forward(self.norm2.forward(h, ctx), ctx, h, **more)
         out, ctx.carry = ctx.carry, None
         return out
+
+
+@BLOCKS.register("sandwich")
+class SandwichBlock(Block):
+    """h += norm1b(mixer(norm1(h))); h += norm2b(ffn(norm2(h))): a norm before and after each sublayer.
+    A layer without a feed-forward has the first half only.
+
+    A sublayer's output is normed before it joins the residual stream, so it cannot be added there by the
+    sublayer's last product.  A part that sets `takes_post_norm` is called with `post_norm=(weight, eps)` and
+    ends with one kernel that norms its float32 output rows and adds them; any other part adds into a zeroed
+    float32 buffer in place of the stream, which is then normed and added."""
+    slots = {"norm1": NORMS, "mixer": MIXERS, "norm1b": NORMS, "norm2": NORMS, "ffn": FEED_FORWARDS, "norm2b": NORMS}
+    optional_slots = ("norm2", "ffn", "norm2b")
+
+    def __init__(self, parts: dict, prefixes: dict):
+        self.norm1, self.mixer, self.norm1b = parts["norm1"], parts["mixer"], parts["norm1b"]
+        self.ffn = parts.get("ffn")
+        self.norm2, self.norm2b = parts.get("norm2"), parts.get("norm2b")
+        if self.ffn is not None and (self.norm2 is None or self.norm2b is None):
+            raise ValueError("a sandwich block with a feed-forward needs norm2 and norm2b")
+        self._prefixes = prefixes
+
+    def children(self):
+        return [(self._prefixes[s], getattr(self, s)) for s in self.slots if getattr(self, s, None) is not None]
+
+    @staticmethod
+    def _sublayer(part, post, x, ctx, h, *cache):
+        rms = post.rms_params()
+        if rms is not None and getattr(part, "takes_post_norm", False):
+            part.forward(x, ctx, *cache, h, post_norm=rms)
+            return
+        from .. import ops
+        out = torch.empty_like(h)
+        ops.fill_u32(out, 0)
+        part.forward(x, ctx, *cache, out)
+        debug.region("norm")
+        if rms is not None:
+            ops.rmsnorm_add(h, out, rms[0], rms[1])
+        else:
+            ops.residual_add(h, post.forward(out, ctx))
+
+    def forward(self, h, ctx, cache):
+        debug.region("norm")
+        self._sublayer(self.mixer, self.norm1b, self.norm1.forward(h, ctx), ctx, h, cache)
+        if self.ffn is not None:
+            debug.region("norm")
+            self._sublayer(self.ffn, self.norm2b, self.norm2.forward(h, ctx), ctx, h)

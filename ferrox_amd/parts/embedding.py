@@ -12,15 +12,16 @@ from .linear import matmul
 class TokenEmbedding(Part):
     kernel_libraries = ("elementwise",)
 
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, name: str = "weight"):
         self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.name = name
         self.weight = None
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.vocab_size, self.hidden_size))}
+        return {self.name: ParamSpec((self.vocab_size, self.hidden_size))}
 
     def load(self, fetch):
-        self.weight = fetch("weight").contiguous()
+        self.weight = fetch(self.name).contiguous()
 
     def forward(self, token_ids):
         return ops.embed(self.weight, token_ids)

@@ -248,3 +248,89 @@ class SparseMoE(FeedForward):
         else:
             ops.moe_combine(residual, y, None, weights, self.top_k)
             self.shared.forward(x, ctx, residual, row_scale=gate)
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExperts(FeedForward):
+    """A mixture of ungated experts, down_e(act(up_e x)), whose router may have more outputs than there are
+    experts: the last `n_identity` outputs are identity experts, which hand the input row through.  The k
+    outputs with the largest score (+ a per-output selection bias, if the model has one) are chosen; the
+    mixture's weights are the scores themselves, divided by their sum only if `renorm`."""
+    kernel_libraries = ("elementwise", "gemm", "moe")
+    takes_post_norm = True
+    TENSORS = {"router": "router", "bias": "correction", "up": "e{}.up", "down": "e{}.down"}
+
+    def __init__(self, hidden_size: int, n_experts: int, top_k: int, expert_intermediate_size: int, n_identity: int = 0,
+                 activation: str = "relu2", gating: str = "softmax", renorm: bool = False, selection_bias: bool = False,
+                 names: dict | None = None):
+        n_out = int(n_experts) + int(n_identity)
+        if n_experts < 0 or n_identity < 0 or not 1 <= top_k <= n_out:
+            raise ValueError(f"top_k {top_k} of {n_experts} experts and {n_identity} identity experts")
+        if n_out > limits.MOE_MAX_EXPERTS or top_k > limits.MOE_MAX_TOP_K:
+            raise ValueError(f"{n_out} router outputs / top_k {top_k}: the routing kernels take up to "
+                             f"{limits.MOE_MAX_EXPERTS} and {limits.MOE_MAX_TOP_K} per token")
+        if gating not in GATINGS:
+            raise ValueError(f"gating '{gating}' is not one of {sorted(GATINGS)}")
+        if activation not in ops.STORED_ACTIVATIONS or activation is None:
+            raise ValueError(f"activation '{activation}' is not one of {sorted(a for a in ops.STORED_ACTIVATIONS if a)}")
+        self.hidden_size, self.n_experts, self.n_identity, self.top_k = int(hidden_size), int(n_experts), int(n_identity), int(top_k)
+        self.expert_intermediate_size = int(expert_intermediate_size)
+        self.activation, self.gating, self.renorm = activation, GATINGS[gating], bool(renorm)
+        self.has_bias = bool(selection_bias)
+        self.names = dict(self.TENSORS, **(names or {}))
+        self.router = self.bias = self.w_up = self.w_down = None
+        self.kblocked = False
+
+    def param_specs(self):
+        H, I, n = self.hidden_size, self.expert_intermediate_size, self.names
+        specs = {n["router"]: ParamSpec((self.n_experts + self.n_identity, H))}
+        if self.has_bias:
+            specs[n["bias"]] = ParamSpec((self.n_experts + self.n_identity,))
+        for e in range(self.n_experts):
+            specs[n["up"].format(e)] = ParamSpec((I, H))
+            specs[n["down"].format(e)] = ParamSpec((H, I))
+        return specs
+
+    def load(self, fetch):
+        n, H, I = self.names, self.hidden_size, self.expert_intermediate_size
+        self.router = fetch(n["router"]).contiguous()
+        self.bias = fetch(n["bias"]).float().contiguous() if self.has_bias else None
+        if self.n_experts:
+            up = torch.stack(same_dtype([fetch(n["up"].format(e)) for e in range(self.n_experts)])).contiguous()     # [E, I, H]
+            down = torch.stack(same_dtype([fetch(n["down"].format(e)) for e in range(self.n_experts)])).contiguous()  # [E, H, I]
+            self.kblocked = up.dtype == torch.bfloat16 and down.dtype == torch.bfloat16 and H % 64 == 0 and I % 64 == 0
+            if self.kblocked:       # streamed weights are kept in slabs of 64 k where the kernels take that
+                up, down = ops.to_kblocked(up), ops.to_kblocked(down)
+            self.w_up, self.w_down = up, down
+
+    def forward(self, x, ctx, residual, post_norm=None) -> None:
+        T, k, E = x.shape[0], self.top_k, self.n_experts
+        debug.region("router")
+        logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
+        ids, weights, _ = ops.router_select(logits, E + self.n_identity, k, self.renorm, self.gating, False,
+                                            selection_bias=self.bias)
+        if debug.routing_trace is not None:
+            debug.routing_trace.put(ids)
+        y = None
+        if E:
+            kb = dict(w_kblocked=True) if self.kblocked else {}
+            H, I = self.hidden_size, self.expert_intermediate_size
+            unsorted = (T <= 16 and T * k <= 64 and x.dtype == torch.bfloat16 and self.w_up.dtype == torch.bfloat16
+                        and H % 8 == 0 and I % 8 == 0)
+            if unsorted:       # few pairs: the products group them by expert themselves (pairs of identity experts are skipped)
+                debug.region("experts up")
+                act = ops.gemm(x, self.w_up, epilogue=ops.EPI_STORE, store_activation=self.activation, pair_ids=ids,
+                               pair_div=k, **kb)
+                debug.region("experts down")
+                y = ops.gemm(act, self.w_down, epilogue=ops.EPI_STORE_F32, pair_ids=ids, **kb)
+            else:              # sorted by router output: the identity experts' pairs come last and belong to no product
+                offsets, sorted_token, sorted_pair, _ = ops.moe_align(ids, E + self.n_identity)
+                debug.region("experts up")
+                act = matmul(x, self.w_up, epilogue=ops.EPI_STORE, store_activation=self.activation, a_rows=sorted_token,
+                             expert_offsets=offsets, n_rows=T * k, **kb)
+                debug.region("experts down")
+                y = matmul(act, self.w_down, epilogue=ops.EPI_STORE_F32, expert_offsets=offsets, c_rows=sorted_pair, **kb)
+        else:
+            y = torch.empty((T * k, self.hidden_size), dtype=torch.float32, device=x.device)
+        debug.region("combine")
+        ops.moe_combine_identity(residual, y, ids, weights, x, E, post_norm)

@@ -10,16 +10,18 @@ from .base import NORMS, Norm, ParamSpec
 class RMSNorm(Norm):
     kernel_libraries = ("elementwise",)
 
-    def __init__(self, size: int, eps: float):
+    def __init__(self, size: int, eps: float, name: str = "weight"):
+        """`name`: what the weight is called behind the part's prefix."""
         self.size = int(size)
         self.eps = float(eps)
+        self.name = name
         self.weight = None
 
     def param_specs(self):
-        return {"weight": ParamSpec((self.size,), init="ones")}
+        return {self.name: ParamSpec((self.size,), init="ones")}
 
     def load(self, fetch):
-        self.weight = fetch("weight").contiguous()
+        self.weight = fetch(self.name).contiguous()
 
     def rms_params(self):
         return self.weight, self.eps

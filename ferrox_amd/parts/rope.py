@@ -44,3 +44,44 @@ class NoPositions(PositionEncoding):
 
     def rotary(self):
         return Rotary(0, 1.0)
+
+
+def scaled_frequencies(rotary_dim: int, theta: float, scaling) -> tuple:
+    """theta^(-2i/rotary_dim) with a wavelength-dependent correction, in float64.  `scaling` = (factor, low, high,
+    original): with L = 2 pi / f the wavelength of a pair, f is kept where L < original / high, divided by `factor`
+    where L > original / low, and blended in between, (1 - s) f / factor + s f with
+    s = (original / L - low) / (high - low): short waves keep their resolution, long ones are stretched to a
+    context `factor` times the original one."""
+    import math
+    out = []
+    for i in range(rotary_dim // 2):
+        f = float(theta) ** (-2.0 * i / rotary_dim)
+        if scaling is not None:
+            factor, low, high, original = (float(x) for x in scaling)
+            wavelength = 2.0 * math.pi / f
+            if wavelength > original / low:
+                f = f / factor
+            elif wavelength >= original / high:
+                s = (original / wavelength - low) / (high - low)
+                f = (1.0 - s) * f / factor + s * f
+        out.append(f)
+    return tuple(out)
+
+
+@POSITION_ENCODINGS.register("rope_scaled")
+class ScaledRope(_Rotary):
+    """A rotation whose frequencies are a table of this part's own (`scaled_frequencies`); either pairing."""
+
+    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None, interleaved: bool = False,
+                 scaling=None):
+        super().__init__(head_dim, theta, rotary_dim)
+        self.interleaved = bool(interleaved)
+        if scaling is not None:
+            scaling = tuple(float(x) for x in scaling)
+            if len(scaling) != 4 or min(scaling) <= 0 or not scaling[2] > scaling[1]:
+                raise ValueError(f"rope scaling is (factor, low, high, original), all positive, high > low; got {scaling}")
+        self.scaling = scaling
+        self.frequencies = scaled_frequencies(self.rotary_dim, self.theta, scaling)
+
+    def rotary(self):
+        return Rotary(self.rotary_dim, self.theta, self.interleaved, None, self.frequencies)

@@ -80,7 +80,11 @@ def test_stop_ids_are_one_or_several():
 
 
 def test_registry_is_closed(tmp_path):
-    assert known_architectures() == ["Qwen2MoeForCausalLM"]
+    assert known_architectures() == ["Qwen2MoeForCausalLM", "Rafilix"]
+    assert resolve({"architecture": "Rafilix"}).model_type == "rafilix"
+    with pytest.raises(ConfigError) as e:
+        resolve({"architecture": "Rafilux"})
+    assert "Rafilux" in str(e.value)
     assert resolve({"architectures": ["Qwen2MoeForCausalLM"]}).model_type == "qwen2_moe"
     assert resolve({"model_type": "qwen2_moe"}).name == "Qwen2MoeForCausalLM"
     with pytest.raises(ConfigError) as e:
