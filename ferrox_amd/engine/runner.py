@@ -98,7 +98,10 @@ class DecodeGraph:
         self.copied.record()
         model, caches = self.runner.model, self.runner.storage.caches
         if self.graph is None:
-            model.forward(self._context(), caches)              # once eagerly: loads the kernels
+            # This step runs eagerly (which also loads the kernels), then the same launches are recorded for the
+            # steps to come.  Recording executes nothing, and the recorded step is not replayed now: a mixer that
+            # carries state from token to token must see every token once.
+            first = model.forward(self._context(), caches)
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             # no garbage collection while the stream is recording: a tensor of an earlier step that is freed
@@ -126,6 +129,7 @@ class DecodeGraph:
             self.graph = graph
             if debug.routing_trace is not None:
                 self.trace_calls = debug.routing_trace.calls()
+            return first[:len(entries)]
         self.graph.replay()
         if debug.routing_trace is not None:
             debug.routing_trace.replayed(self.trace_calls)
