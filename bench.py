@@ -405,6 +405,98 @@ def run_workload(name: str, args) -> int:
     return 0
 
 
+# ---- Rafilix beside the closest existing model, at equal layer sizes ------------------------------------------------
+# Layer sizes that resemble a real model's; every model is four layers of random weights.  The Rafilix layers are
+# measured by kind (all attention, all recurrent) and in the design's usual mixture, the Qwen2-MoE layers have the
+# same width, heads, experts and expert width and no shared expert (Rafilix has none).
+DESIGN_SIZES = {
+    "1k": dict(width=1024, heads=8, kv_heads=2, dim=128, experts=16, identity=2, top=2, ff=704, vocab=32000),
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, experts=60, identity=4, top=4, ff=1408, vocab=32000),
+}
+
+
+def design_configs(s: dict) -> dict:
+    mlp = {"kind": "moe", "expert": {"ff": s["ff"]}, "router": {"experts": s["experts"], "identity": s["identity"], "top": s["top"]}}
+    attn = {"type": "attention", "mlp": mlp, "mixer": {
+        "heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5,
+        "mask": {"size": 8192}, "rot": {"base": 500000.0, "dims": s["dim"],
+                                        "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}}
+    delta = {"type": "channel_delta", "mlp": mlp, "mixer": {
+        "heads": s["heads"], "kv_heads": s["heads"], "dim": s["dim"], "vdim": s["dim"], "conv": 4,
+        "decay_rank": s["dim"], "gate_rank": s["dim"]}}
+
+    def rafilix(layers):
+        return {"architecture": "Rafilix", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "layers": layers,
+                "max_positions": 16384}
+    qwen = dict(A27B, hidden_size=s["width"], num_attention_heads=s["heads"], num_key_value_heads=s["kv_heads"],
+                head_dim=s["dim"], num_experts=s["experts"], num_experts_per_tok=s["top"], moe_intermediate_size=s["ff"],
+                shared_expert_intermediate_size=0, vocab_size=s["vocab"], num_hidden_layers=4, max_position_embeddings=16384,
+                tie_word_embeddings=True)
+    return {"qwen2-moe": qwen, "rafilix attention": rafilix([attn] * 4), "rafilix recurrent": rafilix([delta] * 4),
+            "rafilix mixed": rafilix([attn, delta, delta, attn])}
+
+
+def compare_designs(args) -> int:
+    import torch
+    from ferrox_amd.engine.loading import random_model
+    from ferrox_amd.engine.runner import ModelRunner, StepEntry
+    rng = random.Random(99)
+    results = []
+    sizes = [args.design_size] if args.design_size else sorted(DESIGN_SIZES)
+    for size in sizes:
+        s = DESIGN_SIZES[size]
+        for name, cfg in design_configs(s).items():
+            if args.design and args.design not in name:
+                continue
+            model = random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
+            bs, T, B = args.block_size, args.ctx, args.batch
+            runner = ModelRunner(model, block_size=bs, num_pages=(B + 1) * (-(-(T + args.steps + args.warmup + 2) // bs)) + 8,
+                                 max_seqs=B + 1)
+            V = s["vocab"]
+
+            def prompt(n):
+                return [rng.randrange(V) for _ in range(n)]
+            times = []
+            for rep in range(4):                                   # prefill of one prompt; the first run is thrown away
+                toks = prompt(T)
+                assert runner.admit("p") and runner.reserve("p", T)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                runner.step([StepEntry("p", toks, [T - 1])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                runner.release("p")
+            r = {"size": size, "design": name, "layers": 4, "dtype": args.dtype, "prefill_tokens": T,
+                 "prefill_ms": round(1e3 * statistics.median(times[1:]), 3),
+                 "prefill_tokens_per_s": round(T / statistics.median(times[1:]), 1)}
+            ids = [f"d{i}" for i in range(B)]
+            for rid in ids:
+                assert runner.admit(rid) and runner.reserve(rid, T)
+                runner.step([StepEntry(rid, prompt(T), [])])
+            for batch in sorted({1, B}):
+                live = ids[:batch]
+
+                def steps(n):
+                    for _ in range(n):
+                        for rid in live:
+                            assert runner.reserve(rid, 1)
+                        runner.step([StepEntry(rid, [rng.randrange(V)], [0]) for rid in live])
+                steps(args.warmup)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                steps(args.steps)
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) / args.steps
+                r[f"decode_b{batch}_ms_per_step"] = round(1e3 * dt, 4)
+                r[f"decode_b{batch}_tokens_per_s"] = round(batch / dt, 1)
+            log(json.dumps(r))
+            results.append(r)
+            del runner, model
+            torch.cuda.empty_cache()
+    print(json.dumps({"compare_designs": results, "data": "synthetic", "ctx": args.ctx}), flush=True)
+    return 0
+
+
 # ---- per-kernel table (rocprofv3 around a child process) ----------------------------------------------------------
 KERNEL_TABLES = {"decode_b1": ("decode", 1), "decode_b8": ("decode", 8), "decode_b16": ("decode", 16), "decode_b17": ("decode", 17), "decode_b24": ("decode", 24),
                  "decode_b32": ("decode", 32), "decode_b64": ("decode", 64), "decode_b96": ("decode", 96), "decode_b128": ("decode", 128),
@@ -632,11 +724,18 @@ def main() -> int:
     ap.add_argument("--kernel-table", metavar="WHAT", choices=sorted(KERNEL_TABLES),
                     help="per-kernel times of one workload, measured by rocprofv3 around a child process")
     ap.add_argument("--out", help="with --kernel-table: also write the table to this file")
+    ap.add_argument("--compare-designs", action="store_true",
+                    help="Rafilix layers (all attention, all recurrent, mixed) beside Qwen2-MoE layers of equal sizes: "
+                         "prefill of --ctx tokens, decode at batch 1 and --batch; random weights, four layers each")
+    ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), help="with --compare-designs: one size only")
+    ap.add_argument("--design", help="with --compare-designs: only the designs whose name holds this text")
     ap.add_argument("--profile-run", metavar="WHAT", choices=sorted(KERNEL_TABLES), help=argparse.SUPPRESS)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
         return 2
+    if args.compare_designs:
+        return compare_designs(args)
     if args.workload:
         return run_workload(args.workload, args)
     if args.kernel_table:

@@ -141,7 +141,7 @@ class RafilixConfig:
     layers: tuple
     raw: dict = field(default_factory=dict, compare=False, repr=False)
     eos_token_id: int | tuple | None = None
-    max_positions: int = 1 << 20          # the design has no limit of its own; positions are int32 in the kernels
+    max_positions: int = 32768            # the design names no limit; the optional key `max_positions` does (it sizes the default cache)
     defaulted_keys: tuple = field(default=(), compare=False)
 
     architecture = "Rafilix"
@@ -169,7 +169,7 @@ class RafilixConfig:
         if isinstance(eos, list):
             eos = tuple(int(e) for e in eos)
         return cls(vocab, width, eps, tuple(layers), copy.deepcopy(raw), eos,
-                   r.integer("max_positions", 1 << 20, minimum=1), tuple(r.defaulted))
+                   r.integer("max_positions", 32768, minimum=1), tuple(r.defaulted))
 
     def to_dict(self) -> dict:
         out = copy.deepcopy(self.raw)

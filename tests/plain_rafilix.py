@@ -91,9 +91,9 @@ def attention(h: torch.Tensor, w: dict, m: dict, eps: float, first_pos: int = 0,
         g = hd // (H // G)
         for i in range(T):
             js = [j for j in range(T) if chunk_visible(first_pos + i, first_pos + j, size)]
-            s = torch.stack([(q[i, hd] * k[j, g]).sum() for j in js]) * m["scale"]
+            s = (k[js, g] @ q[i, hd]) * m["scale"]          # one score per visible key
             p = torch.softmax(s, dim=0)
-            out[i, hd] = sum(p[n] * v[j, g] for n, j in enumerate(js))
+            out[i, hd] = p @ v[js, g]
     return out.reshape(T, H * V) @ w["o"].T
 
 
@@ -143,20 +143,35 @@ def channel_delta(h: torch.Tensor, w: dict, m: dict, eps: float) -> torch.Tensor
 # --------------------------------------------------------------------------
 # feed-forward
 # --------------------------------------------------------------------------
-def route(h: torch.Tensor, w: dict, r: dict):
+def route(h: torch.Tensor, w: dict, r: dict, chosen=None):
     """ids [T, top] and weights [T, top]: softmax over all router outputs, the `top` largest of
-    (score + correction) chosen, weighted by the score itself."""
+    (score + correction) chosen, weighted by the score itself.  `chosen`: ids to take instead of the
+    router's own choice (the weights are still this router's scores)."""
     s = torch.softmax(h @ w["router"].T, dim=-1)
     choice = s + w["correction"]
-    ids = torch.topk(choice, r["top"], dim=-1).indices
+    ids = torch.topk(choice, r["top"], dim=-1).indices if chosen is None else torch.as_tensor(chosen, dtype=torch.int64)
     return ids, torch.gather(s, 1, ids)
 
 
-def moe(h: torch.Tensor, w: dict, f: dict, routing=None) -> torch.Tensor:
-    """Experts e < experts are down_e(relu(up_e h)^2); router outputs experts .. experts+identity-1 hand h through."""
+def choice_margin(h: torch.Tensor, w: dict, r: dict, ids) -> float:
+    """How far `ids` are from being the router's top choices: the largest amount by which a choice score that
+    was left out exceeds one that was taken (0 or less: `ids` are a valid top set)."""
+    s = torch.softmax(h @ w["router"].T, dim=-1) + w["correction"]
+    ids = torch.as_tensor(ids, dtype=torch.int64)
+    taken = torch.zeros_like(s, dtype=torch.bool).scatter_(1, ids, True)
+    worst_taken = torch.where(taken, s, torch.full_like(s, float("inf"))).min(dim=-1).values
+    best_left = torch.where(taken, torch.full_like(s, float("-inf")), s).max(dim=-1).values
+    return float((best_left - worst_taken).max())
+
+
+def moe(h: torch.Tensor, w: dict, f: dict, routing=None, margins=None) -> torch.Tensor:
+    """`routing`: the ids [T, top] to use instead of the router's own choice (`margins`, a list, then receives how
+    far they are from it).  Experts e < experts are down_e(relu(up_e h)^2); router outputs experts .. experts+identity-1 hand h through."""
     r = f["router"]
     E = r["experts"]
-    ids, weights = routing if routing is not None else route(h, w, r)
+    ids, weights = route(h, w, r, routing)
+    if routing is not None and margins is not None:
+        margins.append(choice_margin(h, w, r, routing))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for j in range(ids.shape[1]):
@@ -178,12 +193,14 @@ def sub(weights: dict, prefix: str) -> dict:
 
 
 def forward(cfg: dict, weights: dict, tokens: list, dtype=torch.float64, angles: str = "float32", layers_out=None,
-            routing=None):
+            routing=None, margins=None):
     """Logits [T, vocab] of one sequence from position 0.  `layers_out`: a list that receives the residual
-    stream after every layer.  `routing`: per layer (ids, weights) to use instead of the router's own."""
+    stream after every layer.  `routing`: per layer with a feed-forward, in order, the ids [T, top] to use instead
+    of the router's own choice; `margins` then receives how far each is from that choice."""
     W = {k: (v.to(dtype) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = cfg["norm"]["eps"]
     x = W["embed"][torch.tensor(tokens)]
+    n_ff = 0
     for i, layer in enumerate(cfg["layers"]):
         p = f"l{i}."
         h = rms_norm(x, W[p + "norm1"], eps)
@@ -192,7 +209,8 @@ def forward(cfg: dict, weights: dict, tokens: list, dtype=torch.float64, angles:
         x = x + rms_norm(mix(h, sub(W, p + "mix."), layer["mixer"], eps, **kw), W[p + "norm1b"], eps)
         if layer.get("mlp"):
             h = rms_norm(x, W[p + "norm2"], eps)
-            y = moe(h, sub(W, p + "mlp."), layer["mlp"], routing[i] if routing else None)
+            y = moe(h, sub(W, p + "mlp."), layer["mlp"], routing[n_ff] if routing else None, margins)
+            n_ff += 1
             x = x + rms_norm(y, W[p + "norm2b"], eps)
         if layers_out is not None:
             layers_out.append(x.clone())
