@@ -122,107 +122,164 @@ FX_API int fx_delta_prepare(void* stream, const float* q, long ldq, const float*
 // ---------------------------------------------------------------------------
 // The recurrence.  Per head, with S [D, V] carried from token to token:
 //   S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
-// Columns of S never meet, so a block of one wave owns 16 of them: lane (r, j), r = lane / 16, j = lane % 16,
-// holds rows [r DR, (r + 1) DR) of column j in registers (DR = ceil(D / 4) rounded up to the template's size; rows
-// past D stay zero).  Per token it forms, over its rows, the parts of (dS)^T k, (dS)^T q and k.q; the four lanes of
-// a column add theirs with two lane-swapping moves; then u and o = (dS)^T q + u (k.q) follow, and S takes
-// k u^T.  The token's k, q and decay go through LDS (written a token ahead by the wave itself), so every lane
-// reads its rows as broadcasts.  Grid: (ceil(V / 16), heads, sequences).
+// Tokens follow each other, so what bounds a prompt is the time of one token's chain of instructions in one wave;
+// columns of S never meet, so the work is spread over as many waves as that takes: a block of one wave owns
+// 64 / LPC columns, LPC = 16 or 32 lanes to a column.  Lane (c, r), c = lane / LPC, r = lane % LPC, holds rows
+// [r DR, (r + 1) DR) of its column in registers (LPC DR >= D; rows past D stay zero).  Per token it forms, over its
+// rows, the parts of (dS)^T k, (dS)^T q and k.q; the lanes of a column add theirs with four rotations inside their
+// row of 16 lanes and, for 32 lanes, one exchange between neighbouring rows (every lane gets the same bits: each
+// step adds two sums of complementary lanes, and a + b is b + a); then u and o = (dS)^T q + u (k.q) follow, and S
+// takes k u^T.  The tokens' k, q and decay go through LDS, written a group of P tokens ahead by the wave itself
+// (so that memory is waited for once a group, not once a token), and lanes of one r read their rows as broadcasts.
+// The state is kept transposed, [slot][head][V][D]: a lane's rows of its column lie next to each other, and a
+// wave reads and writes contiguous floats (a decode step is little more than that read and write).
+// VEC: D is a multiple of 4, and rows travel in 16-byte pieces.  Grid: (ceil(V / (64 / LPC)), heads, sequences).
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ float column_sum(float x) {      // over lanes j, j + 16, j + 32, j + 48, in each of them
-    const unsigned u = __float_as_uint(x);
-    const auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    const unsigned v = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
-    const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
-    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+template <int LPC>
+__device__ __forceinline__ float column_sum(float v) {      // over the LPC lanes of a column, in each of them
+    v += row_rotated<0x128>(v);      // row_ror:8
+    v += row_rotated<0x124>(v);      // row_ror:4
+    v += row_rotated<0x122>(v);      // row_ror:2
+    v += row_rotated<0x121>(v);      // row_ror:1
+    if constexpr (LPC == 32) {
+        float o;
+        v = wave_partner_16(v, o) + o;      // rows 0 and 1, rows 2 and 3
+    }
+    return v;
 }
 
-template <int DR>
+template <int DR, int LPC, bool VEC>
 __global__ __launch_bounds__(64) void channel_delta_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                                                            const float* __restrict__ decay, const float* __restrict__ beta,
                                                            const float* __restrict__ v, long ldv, float* __restrict__ out, long ldo,
                                                            float* __restrict__ state, const int* __restrict__ seq_starts,
                                                            const int* __restrict__ slots, int H, int G, int D, int V) {
-    constexpr int DP = 4 * DR;                       // rows as the wave holds them
-    __shared__ __attribute__((aligned(16))) float kqd[2][3][DP];      // two tokens x (k, q, decay)
-    const int lane = threadIdx.x, r = lane >> 4, j = blockIdx.x * 16 + (lane & 15);
+    constexpr int DP = LPC * DR;                     // rows as the wave holds them
+    constexpr int W = VEC ? 4 : 1;                   // floats per load
+    constexpr int NF = (3 * DP / W + 63) / 64;       // loads a lane makes per token
+    constexpr int P = NF * W <= 8 ? 8 : 4;           // tokens that travel together
+    constexpr int COLS = 64 / LPC;
+    __shared__ __attribute__((aligned(16))) float kqd[2][P][3][DP];      // two groups of P tokens x (k, q, decay)
+    const int lane = threadIdx.x, r = lane % LPC, j = blockIdx.x * COLS + lane / LPC;
     const int h = blockIdx.y, s = blockIdx.z, g = h / (H / G);
     const int t0 = seq_starts[s], t1 = seq_starts[s + 1];
     if (t1 <= t0) return;
     const bool col = j < V;
-    float* S_g = state + (((size_t)slots[s] * H + h) * D) * V + (col ? j : 0);
+    float* S_g = state + (((size_t)slots[s] * H + h) * V + (col ? j : 0)) * D + r * DR;
     float S[DR];
 #pragma unroll
-    for (int i = 0; i < DR; ++i) {
-        const int row = r * DR + i;
-        S[i] = (col && row < D) ? S_g[(size_t)row * V] : 0.f;
+    for (int i = 0; i < DR; i += 4) {
+        if (VEC) {
+            const bool in = col && r * DR + i < D;      // (D % 4 == 0: a piece is inside or outside as a whole)
+            const float4 x = in ? *(const float4*)(S_g + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+            S[i] = x.x; S[i + 1] = x.y; S[i + 2] = x.z; S[i + 3] = x.w;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) S[i + e] = (col && r * DR + i + e < D) ? S_g[i + e] : 0.f;
+        }
     }
-    // the wave brings a token's k, q and decay into LDS: 3 DP floats, lane-strided; rows past D are zeros
-    auto fetch = [&](int t, float (&buf)[3 * DP / 64 + 1]) {
+    // what this lane brings per token: NF pieces of W floats out of the 3 DP of (k | q | decay); where a piece
+    // comes from is worked out once (a piece past D, or past the three rows, is zeros)
+    const float* src[NF];
+    long step[NF];
+    bool any[NF];
 #pragma unroll
-        for (int n = 0; n < 3 * DP / 64 + 1; ++n) {
-            const int e = n * 64 + lane, which = e / DP, row = e - which * DP;
-            float x = 0.f;
-            if (e < 3 * DP && row < D) {
-                const float* src = which == 0 ? kn + ((size_t)t * G + g) * D : (which == 1 ? qn + ((size_t)t * G + g) * D
-                                                                                             : decay + ((size_t)t * H + h) * D);
-                x = src[row];
+    for (int n = 0; n < NF; ++n) {
+        const int e = (n * 64 + lane) * W, which = e / DP, row = e - which * DP;
+        any[n] = e < 3 * DP && row < D;
+        step[n] = which == 2 ? (long)H * D : (long)G * D;
+        const float* base = which == 0 ? kn + (size_t)g * D : (which == 1 ? qn + (size_t)g * D : decay + (size_t)h * D);
+        src[n] = base + (any[n] ? row : 0) + (size_t)t0 * step[n];
+    }
+    float nxt[P][NF][W], v_nxt[P], b_nxt[P];
+    const float* v_src = v + (size_t)t0 * ldv + (size_t)h * V + (col ? j : 0);
+    const float* b_src = beta + (size_t)t0 * H + h;
+    auto fetch = [&](int first) {                    // tokens first .. first + P - 1 (those before t1)
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            const long dt = first + p - t0;
+            const bool live = first + p < t1;          // (the same in every lane: a group's tokens past the end cost nothing)
+#pragma unroll
+            for (int n = 0; n < NF; ++n) {
+                if (VEC) {
+                    const float4 x = (live && any[n]) ? *(const float4*)(src[n] + dt * step[n]) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    nxt[p][n][0] = x.x; nxt[p][n][W > 1 ? 1 : 0] = x.y; nxt[p][n][W > 1 ? 2 : 0] = x.z; nxt[p][n][W > 1 ? 3 : 0] = x.w;
+                } else {
+                    nxt[p][n][0] = (live && any[n]) ? src[n][dt * step[n]] : 0.f;
+                }
             }
-            buf[n] = x;
+            v_nxt[p] = (live && col) ? v_src[dt * ldv] : 0.f;
+            b_nxt[p] = live ? b_src[dt * H] : 0.f;
         }
     };
-    auto stage = [&](int slot, const float (&buf)[3 * DP / 64 + 1]) {
+    auto stage = [&](int slot) {
 #pragma unroll
-        for (int n = 0; n < 3 * DP / 64 + 1; ++n) {
-            const int e = n * 64 + lane;
-            if (e < 3 * DP) (&kqd[slot][0][0])[e] = buf[n];
-        }
+        for (int p = 0; p < P; ++p)
+#pragma unroll
+            for (int n = 0; n < NF; ++n) {
+                const int e = (n * 64 + lane) * W;
+                if (e < 3 * DP) {
+                    float* dst = &kqd[slot][p][0][0] + e;
+                    if (VEC) *(float4*)dst = make_float4(nxt[p][n][0], nxt[p][n][W > 1 ? 1 : 0], nxt[p][n][W > 1 ? 2 : 0], nxt[p][n][W > 1 ? 3 : 0]);
+                    else *dst = nxt[p][n][0];
+                }
+            }
     };
-    float next[3 * DP / 64 + 1];
-    fetch(t0, next);
-    stage(0, next);
-    float v_next = col ? v[(size_t)t0 * ldv + (size_t)h * V + j] : 0.f, beta_next = beta[(size_t)t0 * H + h];
-    for (int t = t0; t < t1; ++t) {
-        const int cur = (t - t0) & 1;
-        const float vt = v_next, bt = beta_next;
-        if (t + 1 < t1) {                            // the next token's operands leave now and are staged after this token's work
-            fetch(t + 1, next);
-            v_next = col ? v[(size_t)(t + 1) * ldv + (size_t)h * V + j] : 0.f;
-            beta_next = beta[(size_t)(t + 1) * H + h];
+    fetch(t0);
+    stage(0);
+    for (int first = t0, cur = 0; first < t1; first += P, cur ^= 1) {
+        float v_cur[P], b_cur[P];
+#pragma unroll
+        for (int p = 0; p < P; ++p) {
+            v_cur[p] = v_nxt[p];
+            b_cur[p] = b_nxt[p];
         }
+        const bool more = first + P < t1;
+        if (more) fetch(first + P);                  // the next group's operands leave now and are staged after this group's work
         __builtin_amdgcn_wave_barrier();
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // what the wave staged a token ago is in LDS
-        const float* kk = &kqd[cur][0][r * DR];
-        const float* qq = &kqd[cur][1][r * DR];
-        const float* dd = &kqd[cur][2][r * DR];
-        float kv[DR];
-        float sk = 0.f, sq = 0.f, kq = 0.f;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // what the wave staged a group ago is in LDS
 #pragma unroll
-        for (int i = 0; i < DR; i += 4) {
-            const float4 k4 = *(const float4*)(kk + i), q4 = *(const float4*)(qq + i), d4 = *(const float4*)(dd + i);
-            const float ka[4] = {k4.x, k4.y, k4.z, k4.w}, qa[4] = {q4.x, q4.y, q4.z, q4.w}, da[4] = {d4.x, d4.y, d4.z, d4.w};
+        for (int p = 0; p < P; ++p) {
+            const int t = first + p;
+            if (t < t1) {
+                const float* kk = &kqd[cur][p][0][r * DR];
+                const float* qq = &kqd[cur][p][1][r * DR];
+                const float* dd = &kqd[cur][p][2][r * DR];
+                float kv[DR];
+                float sk = 0.f, sq = 0.f, kq = 0.f;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                S[i + e] *= da[e];
-                sk = fmaf(S[i + e], ka[e], sk);
-                sq = fmaf(S[i + e], qa[e], sq);
-                kq = fmaf(ka[e], qa[e], kq);
-                kv[i + e] = ka[e];
+                for (int i = 0; i < DR; i += 4) {
+                    const float4 k4 = *(const float4*)(kk + i), q4 = *(const float4*)(qq + i), d4 = *(const float4*)(dd + i);
+                    const float ka[4] = {k4.x, k4.y, k4.z, k4.w}, qa[4] = {q4.x, q4.y, q4.z, q4.w}, da[4] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        S[i + e] *= da[e];
+                        sk = fmaf(S[i + e], ka[e], sk);
+                        sq = fmaf(S[i + e], qa[e], sq);
+                        kq = fmaf(ka[e], qa[e], kq);
+                        kv[i + e] = ka[e];
+                    }
+                }
+                sk = column_sum<LPC>(sk);
+                sq = column_sum<LPC>(sq);
+                kq = column_sum<LPC>(kq);
+                const float u = b_cur[p] * (v_cur[p] - sk);
+                if (col && r == 0) out[(size_t)t * ldo + (size_t)h * V + j] = fmaf(u, kq, sq);
+#pragma unroll
+                for (int i = 0; i < DR; ++i) S[i] = fmaf(kv[i], u, S[i]);
             }
         }
-        sk = column_sum(sk);
-        sq = column_sum(sq);
-        kq = column_sum(kq);
-        const float u = bt * (vt - sk);
-        if (col && r == 0) out[(size_t)t * ldo + (size_t)h * V + j] = fmaf(u, kq, sq);
-#pragma unroll
-        for (int i = 0; i < DR; ++i) S[i] = fmaf(kv[i], u, S[i]);
-        if (t + 1 < t1) stage(cur ^ 1, next);
+        if (more) stage(cur ^ 1);
     }
 #pragma unroll
-    for (int i = 0; i < DR; ++i) {
-        const int row = r * DR + i;
-        if (col && row < D) S_g[(size_t)row * V] = S[i];
+    for (int i = 0; i < DR; i += 4) {
+        if (VEC) {
+            if (col && r * DR + i < D) *(float4*)(S_g + i) = make_float4(S[i], S[i + 1], S[i + 2], S[i + 3]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col && r * DR + i + e < D) S_g[i + e] = S[i + e];
+        }
     }
 }
 
@@ -234,11 +291,18 @@ FX_API int fx_channel_delta(void* stream, const float* qn, const float* kn, cons
     FX_REQUIRE(ldv >= (long)H * V && ldo >= (long)H * V, "channel_delta: rows of %ld and %ld hold fewer than %d values", ldv, ldo, H * V);
     FX_REQUIRE(n_seqs <= 65535 && H <= 65535, "channel_delta: %d sequences of %d heads are more than a launch takes", n_seqs, H);
     if (n_seqs == 0) return 0;
-    const dim3 grid((V + 15) / 16, H, n_seqs);
+    const bool vec = D % 4 == 0 && (((uintptr_t)state | (uintptr_t)qn | (uintptr_t)kn | (uintptr_t)decay) % 16) == 0;
     hipStream_t s = (hipStream_t)stream;
-    if (D <= 64) channel_delta_kernel<16><<<grid, 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V);
-    else if (D <= 128) channel_delta_kernel<32><<<grid, 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V);
-    else channel_delta_kernel<64><<<grid, 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V);
+#define FX_DELTA(DR_, LPC_)                                                                                                   \
+    do {                                                                                                                      \
+        const dim3 grid((V + 64 / LPC_ - 1) / (64 / LPC_), H, n_seqs);                                                       \
+        if (vec) channel_delta_kernel<DR_, LPC_, true><<<grid, 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V); \
+        else channel_delta_kernel<DR_, LPC_, false><<<grid, 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V);    \
+    } while (0)
+    if (D <= 64) FX_DELTA(4, 16);
+    else if (D <= 128) FX_DELTA(4, 32);
+    else FX_DELTA(8, 32);
+#undef FX_DELTA
     FX_CHECK_LAUNCH("channel_delta");
     return 0;
 }

@@ -770,7 +770,7 @@ def delta_prepare(q, k, a, b, A_log, dt_bias, n_heads: int, n_kv_heads: int, key
 def channel_delta(qn, kn, decay, beta, v, state, seq_starts, slot_ids, n_seqs: int, n_heads: int, n_kv_heads: int,
                   key_dim: int, v_dim: int) -> torch.Tensor:
     """The gated delta rule with a decay per key channel, over each sequence's tokens in order, from and into
-    state[slot] (float32 [slots, H, D, V]):  S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;
+    state[slot] (float32 [slots, H, V, D], the state's transpose: a column's key channels lie together):  S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;
     o_t = S^T q_t.  Returns o float32 [T, H*V]."""
     T = qn.shape[0]
     H, G, D, V = int(n_heads), int(n_kv_heads), int(key_dim), int(v_dim)
@@ -778,8 +778,8 @@ def channel_delta(qn, kn, decay, beta, v, state, seq_starts, slot_ids, n_seqs: i
         if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (T, cols):
             raise KernelError(f"channel_delta: {what} must be contiguous float32 [{T}, {cols}]")
     _f32_rows(v, "channel_delta: v", H * V)
-    if v.shape[0] != T or state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, D, V):
-        raise KernelError(f"channel_delta: v {tuple(v.shape)} / state {tuple(state.shape)} for [slots, {H}, {D}, {V}]")
+    if v.shape[0] != T or state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (H, V, D):
+        raise KernelError(f"channel_delta: v {tuple(v.shape)} / state {tuple(state.shape)} for [slots, {H}, {V}, {D}]")
     if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs:
         raise KernelError("channel_delta: the step's index tensors are shorter than its sequences")
     out = torch.empty((T, H * V), dtype=torch.float32, device=qn.device)

@@ -78,9 +78,9 @@ class PagedAttention(Mixer):
         the two norms among them)."""
         if n_heads % n_kv_heads:
             raise ValueError(f"n_heads {n_heads} is not a multiple of n_kv_heads {n_kv_heads}")
-        if head_dim % limits.HEAD_DIM_STEP or not limits.HEAD_DIM_STEP <= head_dim <= limits.HEAD_DIM_MAX:
-            raise ValueError(f"head_dim {head_dim}: the attention kernels take multiples of {limits.HEAD_DIM_STEP} "
-                             f"up to {limits.HEAD_DIM_MAX}")
+        # (the matrix-unit kernels take multiples of HEAD_DIM_STEP; other sizes run on the kernels for any shape)
+        if not 1 <= head_dim <= limits.HEAD_DIM_MAX:
+            raise ValueError(f"head_dim {head_dim}: the attention kernels take head sizes up to {limits.HEAD_DIM_MAX}")
         self.hidden_size, self.n_heads, self.n_kv_heads, self.head_dim = hidden_size, n_heads, n_kv_heads, head_dim
         self.bias = bool(bias)
         self.window = int(window) if window else None

@@ -89,7 +89,7 @@ class ChannelDelta(Mixer):
 
     def state_shapes(self) -> dict:
         return {"conv": ((self.conv_channels, self.conv_taps - 1), torch.float32),
-                "S": ((self.n_heads, self.key_dim, self.v_dim), torch.float32)}
+                "S": ((self.n_heads, self.v_dim, self.key_dim), torch.float32)}      # kept transposed: [head][value][key]
 
     def forward(self, x, ctx, cache, residual, post_norm=None) -> None:
         H, G, D, V = self.n_heads, self.n_kv_heads, self.key_dim, self.v_dim

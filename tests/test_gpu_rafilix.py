@@ -266,6 +266,18 @@ def test_long_decoding_on_the_matrix_units(tmp_path_factory, dtype):
     run_and_check(u.CFG_MFMA, weights, model, reqs, whole, dtype, "whole", block_size=64, num_pages=8)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_that_fit_no_vector(tmp_path_factory, dtype):
+    """Head sizes, widths and a vocabulary that are no multiples of 16, 8 or 4: the kernels' guarded paths."""
+    cfg = u.config([u.attention_layer(heads=3, kv_heads=3, dim=24, vdim=40, chunk=7, rot_dims=10, scale=0.6, mlp=u.moe(3, 1, 2, 20)),
+                    u.delta_layer(heads=3, kv_heads=1, dim=30, vdim=10, conv=2, mlp=u.moe(2, 2, 1, 12)),
+                    u.attention_layer(heads=2, kv_heads=1, dim=18, vdim=6, chunk=0, rot_dims=18, scale=0.5)], width=70, vocab=151)
+    weights, model = model_for(tmp_path_factory, "odd", cfg, 13, dtype, decay_rank=5, gate_rank=7)
+    reqs = {"a": u.random_tokens(151, 45, 1), "b": u.random_tokens(151, 20, 2)}
+    sched = [[("a", 30), ("b", 2)], [("a", 1), ("b", 17)]] + [[("a", 1), ("b", 1)]] + [[("a", 1)]] * 13
+    run_and_check(cfg, weights, model, reqs, sched, dtype, "odd sizes")
+
+
 def test_pages_of_ended_chunks_are_given_back(tmp_path_factory):
     """A chunked layer needs the pages of the chunk in progress only: with every attention layer chunked, a prompt
     of 200 tokens runs in a pool of 5 pages of 16 (chunks of 40 span at most 4), in portions of at most a chunk."""
