@@ -476,39 +476,50 @@ FX_API int fx_rmsnorm_add(void* stream, float* h, const float* y, const void* w,
 // ---------------------------------------------------------------------------
 // The weighted sum of a token's chosen experts where some router outputs are identity experts:
 //   out[t, :] = sum_j w[t, j] * (ids[t, j] < E ? y[t*k + j, :] : x[t, :])
-// in ascending j; y is float32 [T*k, H] in pair order (rows of identity pairs are never read), x the
+// in ascending j; y is float32 [T*k, H] in pair order (rows of identity pairs are read and dropped), x the
 // feed-forward's input rows.  With norm_w the sum is then normed and added into the stream,
 //   h[t, :] += out[t, :] * rsqrt(mean(out[t]^2) + eps) * norm_w,
 // else it is added as it is.  One block per token; `out` [T, H] keeps the sums between the two passes.
 // ---------------------------------------------------------------------------
-template <typename X>
-__global__ __launch_bounds__(256) void moe_combine_identity_kernel(float* __restrict__ h, float* __restrict__ out,
+template <typename X, int NW>
+__global__ __launch_bounds__(NW * 64) void moe_combine_identity_kernel(float* __restrict__ h, float* __restrict__ out,
                                                                    const float* __restrict__ y, const int* __restrict__ ids,
                                                                    const float* __restrict__ w, const X* __restrict__ x,
                                                                    int E, int H, int k, const void* __restrict__ norm_w,
                                                                    int norm_dtype, float eps) {
-    __shared__ float red[4];
+    __shared__ float red[NW];
     const int t = blockIdx.x;
     const size_t row = (size_t)t * H;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < H; c += 256) {
+    for (int c = threadIdx.x; c < H; c += NW * 64) {
         float acc = 0.f;
         const float xv = to_float(x[row + c]);
-        for (int j = 0; j < k; ++j) {
-            const int e = ids[t * k + j];
-            const float v = e < E ? y[((size_t)t * k + j) * H + c] : xv;
-            acc = fmaf(w[t * k + j], v, acc);
+        for (int j0 = 0; j0 < k; j0 += 4) {
+            // four terms' loads leave together; a row of y is read whatever its pair chose (it is memory of this
+            // call's own, written or not) and dropped afterwards, so that no load waits behind a branch
+            float yv[4], wv[4];
+            int ev[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int j = min(j0 + u, k - 1);
+                ev[u] = ids[t * k + j];
+                wv[u] = w[t * k + j];
+                yv[u] = y[((size_t)t * k + j) * H + c];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (j0 + u < k) acc = fmaf(wv[u], ev[u] < E ? yv[u] : xv, acc);
         }
         out[row + c] = acc;
         ss = fmaf(acc, acc, ss);
     }
     if (!norm_w) {
-        for (int c = threadIdx.x; c < H; c += 256) h[row + c] += out[row + c];      // (each thread reads what it wrote)
+        for (int c = threadIdx.x; c < H; c += NW * 64) h[row + c] += out[row + c];      // (each thread reads what it wrote)
         return;
     }
-    ss = block_sum<4>(ss, red);
+    ss = block_sum<NW>(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
-    for (int c = threadIdx.x; c < H; c += 256) h[row + c] += out[row + c] * scale * load_as_float(norm_w, norm_dtype, c);
+    for (int c = threadIdx.x; c < H; c += NW * 64) h[row + c] += out[row + c] * scale * load_as_float(norm_w, norm_dtype, c);
 }
 
 FX_API int fx_moe_combine_identity(void* stream, float* h, float* out, const float* y, const int* ids, const float* w,
@@ -519,10 +530,16 @@ FX_API int fx_moe_combine_identity(void* stream, float* h, float* out, const flo
     FX_REQUIRE(!norm_w || norm_dtype == FX_F32 || norm_dtype == FX_BF16, "moe_combine_identity: unknown norm weight dtype %d", norm_dtype);
     if (T == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    if (x_dtype == FX_F32)
-        moe_combine_identity_kernel<float><<<T, 256, 0, s>>>(h, out, y, ids, w, (const float*)x, E, H, k, norm_w, norm_dtype, eps);
+    // wide rows get blocks of 16 waves: every thread then has a column or two, and all of a row's loads are in flight at once
+    if (H > 1024) {
+        if (x_dtype == FX_F32)
+            moe_combine_identity_kernel<float, 16><<<T, 1024, 0, s>>>(h, out, y, ids, w, (const float*)x, E, H, k, norm_w, norm_dtype, eps);
+        else
+            moe_combine_identity_kernel<bf16, 16><<<T, 1024, 0, s>>>(h, out, y, ids, w, (const bf16*)x, E, H, k, norm_w, norm_dtype, eps);
+    } else if (x_dtype == FX_F32)
+        moe_combine_identity_kernel<float, 4><<<T, 256, 0, s>>>(h, out, y, ids, w, (const float*)x, E, H, k, norm_w, norm_dtype, eps);
     else
-        moe_combine_identity_kernel<bf16><<<T, 256, 0, s>>>(h, out, y, ids, w, (const bf16*)x, E, H, k, norm_w, norm_dtype, eps);
+        moe_combine_identity_kernel<bf16, 4><<<T, 256, 0, s>>>(h, out, y, ids, w, (const bf16*)x, E, H, k, norm_w, norm_dtype, eps);
     FX_CHECK_LAUNCH("moe_combine_identity");
     return 0;
 }

@@ -77,7 +77,8 @@ FX_API int fx_short_conv(void* stream, const float* x, long ldx, float* y, long 
 //   qn = q / sqrt(sum(q^2) + 1e-6) * D^-1/2,  kn = k / sqrt(sum(k^2) + 1e-6)        per q/k head
 //   decay[h, i] = exp(-exp(A_log[h]) * softplus(a[h, i] + dt_bias[h, i]))             per head and key channel
 //   beta[h] = sigmoid(b[h])
-// One block per token.
+// Blocks (token, part): part p makes 256 of the token's decays and, a wave each, heads 4p .. 4p+3 of q and k (a
+// decode step's few tokens then still spread over many blocks).
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.0f ? x : log1pf(expf(x)); }
 
@@ -86,8 +87,8 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const float* __restr
                                                             const void* __restrict__ A_log, const void* __restrict__ dt_bias, int w_dtype,
                                                             float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ decay,
                                                             float* __restrict__ beta, int H, int G, int D) {
-    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int g = wave; g < 2 * G; g += 4) {          // a wave per head of q (g < G) or of k
+    const int t = blockIdx.x, part = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int g = part * 4 + wave; g < 2 * G; g += 4 * gridDim.y) {          // a wave per head of q (g < G) or of k
         const bool is_q = g < G;
         const float* src = is_q ? q + (size_t)t * ldq + (size_t)g * D : k + (size_t)t * ldk + (size_t)(g - G) * D;
         float* dst = is_q ? qn + ((size_t)t * G + g) * D : kn + ((size_t)t * G + g - G) * D;
@@ -98,13 +99,14 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const float* __restr
         if (is_q) scale *= 1.0f / sqrtf((float)D);
         for (int i = lane; i < D; i += 64) dst[i] = src[i] * scale;
     }
-    for (int idx = threadIdx.x; idx < H * D; idx += 256) {
+    for (int idx = part * 256 + threadIdx.x; idx < H * D; idx += 256 * gridDim.y) {
         const int h = idx / D;
         const float rate = expf(load_as_float(A_log, w_dtype, h));
         const float step = softplus_f(a[(size_t)t * lda + idx] + load_as_float(dt_bias, w_dtype, idx));
         decay[(size_t)t * H * D + idx] = expf(-rate * step);
     }
-    for (int h = threadIdx.x; h < H; h += 256) beta[(size_t)t * H + h] = 1.0f / (1.0f + expf(-b[(size_t)t * ldb + h]));
+    if (part == 0)
+        for (int h = threadIdx.x; h < H; h += 256) beta[(size_t)t * H + h] = 1.0f / (1.0f + expf(-b[(size_t)t * ldb + h]));
 }
 
 FX_API int fx_delta_prepare(void* stream, const float* q, long ldq, const float* k, long ldk, const float* a, long lda,
@@ -113,7 +115,8 @@ FX_API int fx_delta_prepare(void* stream, const float* q, long ldq, const float*
     FX_REQUIRE(T >= 0 && H > 0 && G > 0 && D > 0 && H % G == 0, "delta_prepare: bad sizes T=%d H=%d G=%d D=%d", T, H, G, D);
     FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "delta_prepare: unknown dtype %d", w_dtype);
     if (T == 0) return 0;
-    delta_prepare_kernel<<<T, 256, 0, (hipStream_t)stream>>>(q, ldq, k, ldk, a, lda, b, ldb, A_log, dt_bias, w_dtype, qn, kn,
+    const int parts = (int)fminl(1024, fmaxl((H * (long)D + 255) / 256, (2 * G + 3) / 4));
+    delta_prepare_kernel<<<dim3(T, parts), 256, 0, (hipStream_t)stream>>>(q, ldq, k, ldk, a, lda, b, ldb, A_log, dt_bias, w_dtype, qn, kn,
                                                              decay, beta, H, G, D);
     FX_CHECK_LAUNCH("delta_prepare");
     return 0;
@@ -122,18 +125,20 @@ FX_API int fx_delta_prepare(void* stream, const float* q, long ldq, const float*
 // ---------------------------------------------------------------------------
 // The recurrence.  Per head, with S [D, V] carried from token to token:
 //   S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
-// Tokens follow each other, so what bounds a prompt is the time of one token's chain of instructions in one wave;
-// columns of S never meet, so the work is spread over as many waves as that takes: a block of one wave owns
-// 64 / LPC columns, LPC = 16 or 32 lanes to a column.  Lane (c, r), c = lane / LPC, r = lane % LPC, holds rows
-// [r DR, (r + 1) DR) of its column in registers (LPC DR >= D; rows past D stay zero).  Per token it forms, over its
-// rows, the parts of (dS)^T k, (dS)^T q and k.q; the lanes of a column add theirs with four rotations inside their
-// row of 16 lanes and, for 32 lanes, one exchange between neighbouring rows (every lane gets the same bits: each
-// step adds two sums of complementary lanes, and a + b is b + a); then u and o = (dS)^T q + u (k.q) follow, and S
-// takes k u^T.  The tokens' k, q and decay go through LDS, written a group of P tokens ahead by the wave itself
-// (so that memory is waited for once a group, not once a token), and lanes of one r read their rows as broadcasts.
+// Tokens follow each other; columns of S never meet.  A wave owns 64 / LPC columns, LPC = 16 or 32 lanes to a
+// column: lane (c, r), c = lane / LPC, r = lane % LPC, holds rows [r DR, (r + 1) DR) of its column in registers
+// (LPC DR >= D; rows past D stay zero).  Per token it forms, over its rows, the parts of (dS)^T k, (dS)^T q and
+// k.q; the lanes of a column add theirs with four rotations inside their row of 16 lanes and, for 32 lanes, one
+// exchange between neighbouring rows (every lane gets the same bits: each step adds two sums of complementary
+// lanes, and a + b is b + a); then u and o = (dS)^T q + u (k.q) follow, and S takes k u^T.
+// A token's k, q and decay are the same for every column of a head, and reading them is most of the traffic: a
+// block of NW waves (NW 64 / LPC columns) brings them into LDS once for all its waves, a group of P tokens at a
+// time and a group ahead (memory is waited for once a group, not once a token; one barrier a group), and lanes
+// of one r read their rows as broadcasts.  (A wave that fetched for itself made a layer read 3 GB for a prompt of
+// 2,048 tokens at 16 heads of 128 x 128, and more waves made it slower.)
 // The state is kept transposed, [slot][head][V][D]: a lane's rows of its column lie next to each other, and a
 // wave reads and writes contiguous floats (a decode step is little more than that read and write).
-// VEC: D is a multiple of 4, and rows travel in 16-byte pieces.  Grid: (ceil(V / (64 / LPC)), heads, sequences).
+// VEC: D is a multiple of 4, and rows travel in 16-byte pieces.  Grid: (ceil(V / (NW 64 / LPC)), heads, sequences).
 // ---------------------------------------------------------------------------
 template <int LPC>
 __device__ __forceinline__ float column_sum(float v) {      // over the LPC lanes of a column, in each of them
@@ -148,28 +153,32 @@ __device__ __forceinline__ float column_sum(float v) {      // over the LPC lane
     return v;
 }
 
-template <int DR, int LPC, bool VEC>
-__global__ __launch_bounds__(64) void channel_delta_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
-                                                           const float* __restrict__ decay, const float* __restrict__ beta,
-                                                           const float* __restrict__ v, long ldv, float* __restrict__ out, long ldo,
-                                                           float* __restrict__ state, const int* __restrict__ seq_starts,
-                                                           const int* __restrict__ slots, int H, int G, int D, int V) {
-    constexpr int DP = LPC * DR;                     // rows as the wave holds them
+template <int DR, int LPC, bool VEC, int NW>
+__global__ __launch_bounds__(NW * 64) void channel_delta_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
+                                                                const float* __restrict__ decay, const float* __restrict__ beta,
+                                                                const float* __restrict__ v, long ldv, float* __restrict__ out, long ldo,
+                                                                float* __restrict__ state, const int* __restrict__ seq_starts,
+                                                                const int* __restrict__ slots, int H, int G, int D, int V) {
+    constexpr int DP = LPC * DR;                     // rows as a wave holds them
     constexpr int W = VEC ? 4 : 1;                   // floats per load
-    constexpr int NF = (3 * DP / W + 63) / 64;       // loads a lane makes per token
-    constexpr int P = NF * W <= 8 ? 8 : 4;           // tokens that travel together
+    constexpr int P = 8;                             // tokens that travel together
+    constexpr int NT = NW * 64;
+    constexpr int PIECES = 3 * DP / W;               // loads that bring one token's (k | q | decay)
+    constexpr int NL = (P * PIECES + NT - 1) / NT;   // loads a thread makes per group
     constexpr int COLS = 64 / LPC;
+    static_assert(DR % 4 == 0, "a lane's rows are read from LDS in 16-byte pieces");
     __shared__ __attribute__((aligned(16))) float kqd[2][P][3][DP];      // two groups of P tokens x (k, q, decay)
-    const int lane = threadIdx.x, r = lane % LPC, j = blockIdx.x * COLS + lane / LPC;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int r = lane % LPC, j = (blockIdx.x * NW + wave) * COLS + lane / LPC;
     const int h = blockIdx.y, s = blockIdx.z, g = h / (H / G);
     const int t0 = seq_starts[s], t1 = seq_starts[s + 1];
-    if (t1 <= t0) return;
+    if (t1 <= t0) return;                            // (the same in every thread of the block)
     const bool col = j < V;
     float* S_g = state + (((size_t)slots[s] * H + h) * V + (col ? j : 0)) * D + r * DR;
     float S[DR];
 #pragma unroll
     for (int i = 0; i < DR; i += 4) {
-        if (VEC) {
+        if constexpr (VEC) {
             const bool in = col && r * DR + i < D;      // (D % 4 == 0: a piece is inside or outside as a whole)
             const float4 x = in ? *(const float4*)(S_g + i) : make_float4(0.f, 0.f, 0.f, 0.f);
             S[i] = x.x; S[i + 1] = x.y; S[i + 2] = x.z; S[i + 3] = x.w;
@@ -178,55 +187,45 @@ __global__ __launch_bounds__(64) void channel_delta_kernel(const float* __restri
             for (int e = 0; e < 4; ++e) S[i + e] = (col && r * DR + i + e < D) ? S_g[i + e] : 0.f;
         }
     }
-    // what this lane brings per token: NF pieces of W floats out of the 3 DP of (k | q | decay); where a piece
-    // comes from is worked out once (a piece past D, or past the three rows, is zeros)
-    const float* src[NF];
-    long step[NF];
-    bool any[NF];
+    // a group's operands: piece number idx = n NT + tid of the group's P PIECES goes to kqd[.] at idx W, which is
+    // token idx / PIECES, then k, q or decay, then the row; pieces past D, past the group or past the sequence are zeros
+    float nxt[NL][W], v_nxt[P], b_nxt[P];
+    auto fetch = [&](int first) {
 #pragma unroll
-    for (int n = 0; n < NF; ++n) {
-        const int e = (n * 64 + lane) * W, which = e / DP, row = e - which * DP;
-        any[n] = e < 3 * DP && row < D;
-        step[n] = which == 2 ? (long)H * D : (long)G * D;
-        const float* base = which == 0 ? kn + (size_t)g * D : (which == 1 ? qn + (size_t)g * D : decay + (size_t)h * D);
-        src[n] = base + (any[n] ? row : 0) + (size_t)t0 * step[n];
-    }
-    float nxt[P][NF][W], v_nxt[P], b_nxt[P];
-    const float* v_src = v + (size_t)t0 * ldv + (size_t)h * V + (col ? j : 0);
-    const float* b_src = beta + (size_t)t0 * H + h;
-    auto fetch = [&](int first) {                    // tokens first .. first + P - 1 (those before t1)
+        for (int n = 0; n < NL; ++n) {
+            const int idx = n * NT + tid, p = idx / PIECES, e = (idx - p * PIECES) * W, which = e / DP, row = e - which * DP;
+            const int t = first + p;
+            const bool ok = idx < P * PIECES && t < t1 && row < D;
+            const float* src = which == 0 ? kn + ((size_t)t * G + g) * D : (which == 1 ? qn + ((size_t)t * G + g) * D
+                                                                                         : decay + ((size_t)t * H + h) * D);
+            if constexpr (VEC) {
+                const float4 x = ok ? *(const float4*)(src + row) : make_float4(0.f, 0.f, 0.f, 0.f);
+                nxt[n][0] = x.x; nxt[n][W - 3] = x.y; nxt[n][W - 2] = x.z; nxt[n][W - 1] = x.w;
+            } else {
+                nxt[n][0] = ok ? src[row] : 0.f;
+            }
+        }
 #pragma unroll
         for (int p = 0; p < P; ++p) {
-            const long dt = first + p - t0;
-            const bool live = first + p < t1;          // (the same in every lane: a group's tokens past the end cost nothing)
-#pragma unroll
-            for (int n = 0; n < NF; ++n) {
-                if (VEC) {
-                    const float4 x = (live && any[n]) ? *(const float4*)(src[n] + dt * step[n]) : make_float4(0.f, 0.f, 0.f, 0.f);
-                    nxt[p][n][0] = x.x; nxt[p][n][W > 1 ? 1 : 0] = x.y; nxt[p][n][W > 1 ? 2 : 0] = x.z; nxt[p][n][W > 1 ? 3 : 0] = x.w;
-                } else {
-                    nxt[p][n][0] = (live && any[n]) ? src[n][dt * step[n]] : 0.f;
-                }
-            }
-            v_nxt[p] = (live && col) ? v_src[dt * ldv] : 0.f;
-            b_nxt[p] = live ? b_src[dt * H] : 0.f;
+            const bool live = first + p < t1;
+            v_nxt[p] = (live && col) ? v[(size_t)(first + p) * ldv + (size_t)h * V + j] : 0.f;
+            b_nxt[p] = live ? beta[(size_t)(first + p) * H + h] : 0.f;
         }
     };
     auto stage = [&](int slot) {
 #pragma unroll
-        for (int p = 0; p < P; ++p)
-#pragma unroll
-            for (int n = 0; n < NF; ++n) {
-                const int e = (n * 64 + lane) * W;
-                if (e < 3 * DP) {
-                    float* dst = &kqd[slot][p][0][0] + e;
-                    if (VEC) *(float4*)dst = make_float4(nxt[p][n][0], nxt[p][n][W > 1 ? 1 : 0], nxt[p][n][W > 1 ? 2 : 0], nxt[p][n][W > 1 ? 3 : 0]);
-                    else *dst = nxt[p][n][0];
-                }
+        for (int n = 0; n < NL; ++n) {
+            const int idx = n * NT + tid;
+            if (idx < P * PIECES) {
+                float* dst = &kqd[slot][0][0][0] + (size_t)idx * W;
+                if constexpr (VEC) *(float4*)dst = make_float4(nxt[n][0], nxt[n][W - 3], nxt[n][W - 2], nxt[n][W - 1]);
+                else *dst = nxt[n][0];
             }
+        }
     };
     fetch(t0);
     stage(0);
+    __syncthreads();
     for (int first = t0, cur = 0; first < t1; first += P, cur ^= 1) {
         float v_cur[P], b_cur[P];
 #pragma unroll
@@ -236,44 +235,47 @@ __global__ __launch_bounds__(64) void channel_delta_kernel(const float* __restri
         }
         const bool more = first + P < t1;
         if (more) fetch(first + P);                  // the next group's operands leave now and are staged after this group's work
-        __builtin_amdgcn_wave_barrier();
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // what the wave staged a group ago is in LDS
+        auto token = [&](int p, int t) {
+            const float* kk = &kqd[cur][p][0][r * DR];
+            const float* qq = &kqd[cur][p][1][r * DR];
+            const float* dd = &kqd[cur][p][2][r * DR];
+            float kv[DR];
+            float sk = 0.f, sq = 0.f, kq = 0.f;
 #pragma unroll
-        for (int p = 0; p < P; ++p) {
-            const int t = first + p;
-            if (t < t1) {
-                const float* kk = &kqd[cur][p][0][r * DR];
-                const float* qq = &kqd[cur][p][1][r * DR];
-                const float* dd = &kqd[cur][p][2][r * DR];
-                float kv[DR];
-                float sk = 0.f, sq = 0.f, kq = 0.f;
+            for (int i = 0; i < DR; i += 4) {
+                const float4 k4 = *(const float4*)(kk + i), q4 = *(const float4*)(qq + i), d4 = *(const float4*)(dd + i);
+                const float ka[4] = {k4.x, k4.y, k4.z, k4.w}, qa[4] = {q4.x, q4.y, q4.z, q4.w}, da[4] = {d4.x, d4.y, d4.z, d4.w};
 #pragma unroll
-                for (int i = 0; i < DR; i += 4) {
-                    const float4 k4 = *(const float4*)(kk + i), q4 = *(const float4*)(qq + i), d4 = *(const float4*)(dd + i);
-                    const float ka[4] = {k4.x, k4.y, k4.z, k4.w}, qa[4] = {q4.x, q4.y, q4.z, q4.w}, da[4] = {d4.x, d4.y, d4.z, d4.w};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        S[i + e] *= da[e];
-                        sk = fmaf(S[i + e], ka[e], sk);
-                        sq = fmaf(S[i + e], qa[e], sq);
-                        kq = fmaf(ka[e], qa[e], kq);
-                        kv[i + e] = ka[e];
-                    }
+                for (int e = 0; e < 4; ++e) {
+                    S[i + e] *= da[e];
+                    sk = fmaf(S[i + e], ka[e], sk);
+                    sq = fmaf(S[i + e], qa[e], sq);
+                    kq = fmaf(ka[e], qa[e], kq);
+                    kv[i + e] = ka[e];
                 }
-                sk = column_sum<LPC>(sk);
-                sq = column_sum<LPC>(sq);
-                kq = column_sum<LPC>(kq);
-                const float u = b_cur[p] * (v_cur[p] - sk);
-                if (col && r == 0) out[(size_t)t * ldo + (size_t)h * V + j] = fmaf(u, kq, sq);
-#pragma unroll
-                for (int i = 0; i < DR; ++i) S[i] = fmaf(kv[i], u, S[i]);
             }
+            sk = column_sum<LPC>(sk);
+            sq = column_sum<LPC>(sq);
+            kq = column_sum<LPC>(kq);
+            const float u = b_cur[p] * (v_cur[p] - sk);
+            if (col && r == 0) out[(size_t)t * ldo + (size_t)h * V + j] = fmaf(u, kq, sq);
+#pragma unroll
+            for (int i = 0; i < DR; ++i) S[i] = fmaf(kv[i], u, S[i]);
+        };
+        if (first + P <= t1) {                       // a whole group: one stretch of code, so that a token's LDS reads leave
+#pragma unroll                                       // while the token before it is worked on
+            for (int p = 0; p < P; ++p) token(p, first + p);
+        } else {
+#pragma unroll
+            for (int p = 0; p < P; ++p)
+                if (first + p < t1) token(p, first + p);
         }
-        if (more) stage(cur ^ 1);
+        if (more) stage(cur ^ 1);                    // (the buffer that every wave left before the last barrier)
+        __syncthreads();
     }
 #pragma unroll
     for (int i = 0; i < DR; i += 4) {
-        if (VEC) {
+        if constexpr (VEC) {
             if (col && r * DR + i < D) *(float4*)(S_g + i) = make_float4(S[i], S[i + 1], S[i + 2], S[i + 3]);
         } else {
 #pragma unroll
@@ -293,15 +295,18 @@ FX_API int fx_channel_delta(void* stream, const float* qn, const float* kn, cons
     if (n_seqs == 0) return 0;
     const bool vec = D % 4 == 0 && (((uintptr_t)state | (uintptr_t)qn | (uintptr_t)kn | (uintptr_t)decay) % 16) == 0;
     hipStream_t s = (hipStream_t)stream;
-#define FX_DELTA(DR_, LPC_)                                                                                                   \
+#define FX_DELTA(DR_, LPC_, NW_)                                                                                              \
     do {                                                                                                                      \
-        const dim3 grid((V + 64 / LPC_ - 1) / (64 / LPC_), H, n_seqs);                                                       \
-        if (vec) channel_delta_kernel<DR_, LPC_, true><<<grid, 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V); \
-        else channel_delta_kernel<DR_, LPC_, false><<<grid, 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V);    \
+        const int per_block = NW_ * 64 / LPC_;                                                                                \
+        const dim3 grid((V + per_block - 1) / per_block, H, n_seqs);                                                          \
+        if (vec) channel_delta_kernel<DR_, LPC_, true, NW_><<<grid, NW_ * 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V); \
+        else channel_delta_kernel<DR_, LPC_, false, NW_><<<grid, NW_ * 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V);    \
     } while (0)
-    if (D <= 64) FX_DELTA(4, 16);
-    else if (D <= 128) FX_DELTA(4, 32);
-    else FX_DELTA(8, 32);
+    // (blocks of 16 columns, or of 8 for narrow heads, so that a small model still fills some CUs)
+    if (D <= 64 && V <= 32) FX_DELTA(4, 16, 2);
+    else if (D <= 64) FX_DELTA(4, 16, 4);
+    else if (D <= 128) FX_DELTA(4, 32, 8);
+    else FX_DELTA(8, 32, 8);
 #undef FX_DELTA
     FX_CHECK_LAUNCH("channel_delta");
     return 0;

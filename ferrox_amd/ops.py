@@ -703,7 +703,7 @@ def rmsnorm_add(h: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: flo
 def moe_combine_identity(h, y, ids, weights, x, n_experts: int, post_norm=None) -> None:
     """h[t] += N(sum_j weights[t, j] * (y[t*k + j] if ids[t, j] < n_experts else x[t])), N the RMS norm
     `post_norm` = (weight, eps) or nothing.  y: float32 [T*k, H] in pair order (rows of pairs that chose an
-    identity expert, ids >= n_experts, are never read); x: the feed-forward's input rows [T, H]."""
+    identity expert, ids >= n_experts, are never used: they need not have been written); x: the feed-forward's input rows [T, H]."""
     T, H = h.shape
     k = ids.shape[1]
     if h.dtype != torch.float32 or y.dtype != torch.float32 or weights.dtype != torch.float32 or not h.is_contiguous():

@@ -102,7 +102,7 @@ def test_router_selection_bias_and_identity_kernels():
     y = torch.randn(T * k, H, generator=gen)
     x = torch.randn(T, H, generator=gen)
     y_dev = y.clone()
-    y_dev[(ids.reshape(-1) >= E)] = float("nan")          # rows of identity pairs are never read
+    y_dev[(ids.reshape(-1) >= E)] = float("nan")          # rows of identity pairs are never used
     mixed = torch.zeros(T, H, dtype=torch.float64)
     for t in range(T):
         for j in range(k):
