@@ -82,12 +82,46 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
         from_float(out + (size_t)r * H + c, x[c] * scale * load_as_float(w, w_dtype, c));
 }
 
+// Short rows (the heads of q and k, normed one by one): a wave per row, four rows to a block, the row in registers.
+// The same sums in another order than the block-wide kernel's, so a row is always normed by the same kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_short_kernel(const float* __restrict__ h, const int* __restrict__ rows,
+                                                            const void* __restrict__ w, int w_dtype,
+                                                            T* __restrict__ out, int R, int H, float eps) {
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (r >= R) return;
+    const float* x = h + (size_t)(rows ? rows[r] : r) * H;
+    float xv[4], wv[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = lane + i * 64;
+        xv[i] = c < H ? x[c] : 0.f;
+    }
+    load_strided_as_float<4, 64>(w, w_dtype, lane, H, wv);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss += xv[i] * xv[i];
+    ss = wave_sum(ss);
+    const float scale = 1.0f / sqrtf(ss / (float)H + eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = lane + i * 64;
+        if (c < H) from_float(out + (size_t)r * H + c, xv[i] * scale * wv[i]);
+    }
+}
+
 FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* rows, const void* w,
                       int w_dtype, void* out, int R, int H, float eps) {
     FX_REQUIRE(R >= 0 && H > 0, "rmsnorm: bad sizes R=%d H=%d", R, H);
     FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "rmsnorm: unknown weight dtype %d", w_dtype);
     if (R == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
+    if (H <= 256 && (out_dtype == FX_F32 || out_dtype == FX_BF16)) {
+        if (out_dtype == FX_F32) rmsnorm_short_kernel<float><<<(R + 3) / 4, 256, 0, s>>>(h, rows, w, w_dtype, (float*)out, R, H, eps);
+        else rmsnorm_short_kernel<bf16><<<(R + 3) / 4, 256, 0, s>>>(h, rows, w, w_dtype, (bf16*)out, R, H, eps);
+        FX_CHECK_LAUNCH("rmsnorm");
+        return 0;
+    }
     if (out_dtype == FX_F32)
         rmsnorm_kernel<float><<<R, 256, 0, s>>>(h, rows, w, w_dtype, (float*)out, H, eps);
     else if (out_dtype == FX_BF16)

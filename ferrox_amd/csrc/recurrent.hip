@@ -77,6 +77,7 @@ FX_API int fx_short_conv(void* stream, const float* x, long ldx, float* y, long 
 //   qn = q / sqrt(sum(q^2) + 1e-6) * D^-1/2,  kn = k / sqrt(sum(k^2) + 1e-6)        per q/k head
 //   decay[h, i] = exp(-exp(A_log[h]) * softplus(a[h, i] + dt_bias[h, i]))             per head and key channel
 //   beta[h] = sigmoid(b[h])
+//   kq[g] = kn[g] . qn[g]                                                             per q/k head (the recurrence needs it per token)
 // Blocks (token, part): part p makes 256 of the token's decays and, a wave each, heads 4p .. 4p+3 of q and k (a
 // decode step's few tokens then still spread over many blocks).
 // ---------------------------------------------------------------------------
@@ -86,18 +87,27 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const float* __restr
                                                             const float* __restrict__ a, long lda, const float* __restrict__ b, long ldb,
                                                             const void* __restrict__ A_log, const void* __restrict__ dt_bias, int w_dtype,
                                                             float* __restrict__ qn, float* __restrict__ kn, float* __restrict__ decay,
-                                                            float* __restrict__ beta, int H, int G, int D) {
+                                                            float* __restrict__ beta, float* __restrict__ kq, int H, int G, int D) {
     const int t = blockIdx.x, part = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int g = part * 4 + wave; g < 2 * G; g += 4 * gridDim.y) {          // a wave per head of q (g < G) or of k
-        const bool is_q = g < G;
-        const float* src = is_q ? q + (size_t)t * ldq + (size_t)g * D : k + (size_t)t * ldk + (size_t)(g - G) * D;
-        float* dst = is_q ? qn + ((size_t)t * G + g) * D : kn + ((size_t)t * G + g - G) * D;
-        float ss = 0.f;
-        for (int i = lane; i < D; i += 64) ss = fmaf(src[i], src[i], ss);
-        ss = wave_sum(ss);
-        float scale = 1.0f / sqrtf(ss + 1e-6f);
-        if (is_q) scale *= 1.0f / sqrtf((float)D);
-        for (int i = lane; i < D; i += 64) dst[i] = src[i] * scale;
+    for (int g = part * 4 + wave; g < G; g += 4 * gridDim.y) {          // a wave per head of q and k
+        const float* qs = q + (size_t)t * ldq + (size_t)g * D;
+        const float* ks = k + (size_t)t * ldk + (size_t)g * D;
+        float sq = 0.f, sk = 0.f;
+        for (int i = lane; i < D; i += 64) {
+            sq = fmaf(qs[i], qs[i], sq);
+            sk = fmaf(ks[i], ks[i], sk);
+        }
+        const float q_scale = 1.0f / sqrtf(wave_sum(sq) + 1e-6f) * (1.0f / sqrtf((float)D));
+        const float k_scale = 1.0f / sqrtf(wave_sum(sk) + 1e-6f);
+        float dot = 0.f;
+        for (int i = lane; i < D; i += 64) {
+            const float qv = qs[i] * q_scale, kv = ks[i] * k_scale;
+            qn[((size_t)t * G + g) * D + i] = qv;
+            kn[((size_t)t * G + g) * D + i] = kv;
+            dot = fmaf(kv, qv, dot);
+        }
+        dot = wave_sum(dot);
+        if (lane == 0) kq[(size_t)t * G + g] = dot;
     }
     for (int idx = part * 256 + threadIdx.x; idx < H * D; idx += 256 * gridDim.y) {
         const int h = idx / D;
@@ -111,13 +121,13 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(const float* __restr
 
 FX_API int fx_delta_prepare(void* stream, const float* q, long ldq, const float* k, long ldk, const float* a, long lda,
                             const float* b, long ldb, const void* A_log, const void* dt_bias, int w_dtype, float* qn,
-                            float* kn, float* decay, float* beta, int T, int H, int G, int D) {
+                            float* kn, float* decay, float* beta, float* kq, int T, int H, int G, int D) {
     FX_REQUIRE(T >= 0 && H > 0 && G > 0 && D > 0 && H % G == 0, "delta_prepare: bad sizes T=%d H=%d G=%d D=%d", T, H, G, D);
     FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "delta_prepare: unknown dtype %d", w_dtype);
     if (T == 0) return 0;
-    const int parts = (int)fminl(1024, fmaxl((H * (long)D + 255) / 256, (2 * G + 3) / 4));
+    const int parts = (int)fminl(1024, fmaxl((H * (long)D + 255) / 256, (G + 3) / 4));
     delta_prepare_kernel<<<dim3(T, parts), 256, 0, (hipStream_t)stream>>>(q, ldq, k, ldk, a, lda, b, ldb, A_log, dt_bias, w_dtype, qn, kn,
-                                                             decay, beta, H, G, D);
+                                                             decay, beta, kq, H, G, D);
     FX_CHECK_LAUNCH("delta_prepare");
     return 0;
 }
@@ -127,8 +137,8 @@ FX_API int fx_delta_prepare(void* stream, const float* q, long ldq, const float*
 //   S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
 // Tokens follow each other; columns of S never meet.  A wave owns 64 / LPC columns, LPC = 16 or 32 lanes to a
 // column: lane (c, r), c = lane / LPC, r = lane % LPC, holds rows [r DR, (r + 1) DR) of its column in registers
-// (LPC DR >= D; rows past D stay zero).  Per token it forms, over its rows, the parts of (dS)^T k, (dS)^T q and
-// k.q; the lanes of a column add theirs with four rotations inside their row of 16 lanes and, for 32 lanes, one
+// (LPC DR >= D; rows past D stay zero).  Per token it forms, over its rows, the parts of (dS)^T k and (dS)^T q
+// (k.q comes with the token, from the kernel above); the lanes of a column add theirs with four rotations inside their row of 16 lanes and, for 32 lanes, one
 // exchange between neighbouring rows (every lane gets the same bits: each step adds two sums of complementary
 // lanes, and a + b is b + a); then u and o = (dS)^T q + u (k.q) follow, and S takes k u^T.
 // A token's k, q and decay are the same for every column of a head, and reading them is most of the traffic: a
@@ -156,7 +166,7 @@ __device__ __forceinline__ float column_sum(float v) {      // over the LPC lane
 template <int DR, int LPC, bool VEC, int NW>
 __global__ __launch_bounds__(NW * 64) void channel_delta_kernel(const float* __restrict__ qn, const float* __restrict__ kn,
                                                                 const float* __restrict__ decay, const float* __restrict__ beta,
-                                                                const float* __restrict__ v, long ldv, float* __restrict__ out, long ldo,
+                                                                const float* __restrict__ kq_all, const float* __restrict__ v, long ldv, float* __restrict__ out, long ldo,
                                                                 float* __restrict__ state, const int* __restrict__ seq_starts,
                                                                 const int* __restrict__ slots, int H, int G, int D, int V) {
     constexpr int DP = LPC * DR;                     // rows as a wave holds them
@@ -189,7 +199,7 @@ __global__ __launch_bounds__(NW * 64) void channel_delta_kernel(const float* __r
     }
     // a group's operands: piece number idx = n NT + tid of the group's P PIECES goes to kqd[.] at idx W, which is
     // token idx / PIECES, then k, q or decay, then the row; pieces past D, past the group or past the sequence are zeros
-    float nxt[NL][W], v_nxt[P], b_nxt[P];
+    float nxt[NL][W], v_nxt[P], b_nxt[P], kq_nxt[P];
     auto fetch = [&](int first) {
 #pragma unroll
         for (int n = 0; n < NL; ++n) {
@@ -210,6 +220,7 @@ __global__ __launch_bounds__(NW * 64) void channel_delta_kernel(const float* __r
             const bool live = first + p < t1;
             v_nxt[p] = (live && col) ? v[(size_t)(first + p) * ldv + (size_t)h * V + j] : 0.f;
             b_nxt[p] = live ? beta[(size_t)(first + p) * H + h] : 0.f;
+            kq_nxt[p] = live ? kq_all[(size_t)(first + p) * G + g] : 0.f;
         }
     };
     auto stage = [&](int slot) {
@@ -227,11 +238,12 @@ __global__ __launch_bounds__(NW * 64) void channel_delta_kernel(const float* __r
     stage(0);
     __syncthreads();
     for (int first = t0, cur = 0; first < t1; first += P, cur ^= 1) {
-        float v_cur[P], b_cur[P];
+        float v_cur[P], b_cur[P], kq_cur[P];
 #pragma unroll
         for (int p = 0; p < P; ++p) {
             v_cur[p] = v_nxt[p];
             b_cur[p] = b_nxt[p];
+            kq_cur[p] = kq_nxt[p];
         }
         const bool more = first + P < t1;
         if (more) fetch(first + P);                  // the next group's operands leave now and are staged after this group's work
@@ -240,7 +252,7 @@ __global__ __launch_bounds__(NW * 64) void channel_delta_kernel(const float* __r
             const float* qq = &kqd[cur][p][1][r * DR];
             const float* dd = &kqd[cur][p][2][r * DR];
             float kv[DR];
-            float sk = 0.f, sq = 0.f, kq = 0.f;
+            float sk = 0.f, sq = 0.f;
 #pragma unroll
             for (int i = 0; i < DR; i += 4) {
                 const float4 k4 = *(const float4*)(kk + i), q4 = *(const float4*)(qq + i), d4 = *(const float4*)(dd + i);
@@ -250,15 +262,13 @@ __global__ __launch_bounds__(NW * 64) void channel_delta_kernel(const float* __r
                     S[i + e] *= da[e];
                     sk = fmaf(S[i + e], ka[e], sk);
                     sq = fmaf(S[i + e], qa[e], sq);
-                    kq = fmaf(ka[e], qa[e], kq);
                     kv[i + e] = ka[e];
                 }
             }
             sk = column_sum<LPC>(sk);
             sq = column_sum<LPC>(sq);
-            kq = column_sum<LPC>(kq);
             const float u = b_cur[p] * (v_cur[p] - sk);
-            if (col && r == 0) out[(size_t)t * ldo + (size_t)h * V + j] = fmaf(u, kq, sq);
+            if (col && r == 0) out[(size_t)t * ldo + (size_t)h * V + j] = fmaf(u, kq_cur[p], sq);
 #pragma unroll
             for (int i = 0; i < DR; ++i) S[i] = fmaf(kv[i], u, S[i]);
         };
@@ -286,7 +296,7 @@ __global__ __launch_bounds__(NW * 64) void channel_delta_kernel(const float* __r
 }
 
 FX_API int fx_channel_delta(void* stream, const float* qn, const float* kn, const float* decay, const float* beta,
-                            const float* v, long ldv, float* out, long ldo, float* state, const int* seq_starts,
+                            const float* kq, const float* v, long ldv, float* out, long ldo, float* state, const int* seq_starts,
                             const int* slots, int n_seqs, int H, int G, int D, int V) {
     FX_REQUIRE(n_seqs >= 0 && H > 0 && G > 0 && H % G == 0, "channel_delta: bad sizes sequences=%d H=%d G=%d", n_seqs, H, G);
     FX_REQUIRE(D >= 1 && D <= 256 && V >= 1, "channel_delta: key size %d (up to 256) and value size %d", D, V);
@@ -299,8 +309,8 @@ FX_API int fx_channel_delta(void* stream, const float* qn, const float* kn, cons
     do {                                                                                                                      \
         const int per_block = NW_ * 64 / LPC_;                                                                                \
         const dim3 grid((V + per_block - 1) / per_block, H, n_seqs);                                                          \
-        if (vec) channel_delta_kernel<DR_, LPC_, true, NW_><<<grid, NW_ * 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V); \
-        else channel_delta_kernel<DR_, LPC_, false, NW_><<<grid, NW_ * 64, 0, s>>>(qn, kn, decay, beta, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V);    \
+        if (vec) channel_delta_kernel<DR_, LPC_, true, NW_><<<grid, NW_ * 64, 0, s>>>(qn, kn, decay, beta, kq, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V); \
+        else channel_delta_kernel<DR_, LPC_, false, NW_><<<grid, NW_ * 64, 0, s>>>(qn, kn, decay, beta, kq, v, ldv, out, ldo, state, seq_starts, slots, H, G, D, V);    \
     } while (0)
     // (blocks of 16 columns, or of 8 for narrow heads, so that a small model still fills some CUs)
     if (D <= 64 && V <= 32) FX_DELTA(4, 16, 2);

@@ -70,9 +70,9 @@ _sigs = {
     ("recurrent", "fx_short_conv"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_int, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_int],
     ("recurrent", "fx_delta_prepare"): [c_void_p, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long, c_void_p, c_long,
-                                        c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int, c_int, c_int, c_int],
-    ("recurrent", "fx_channel_delta"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long,
+    ("recurrent", "fx_channel_delta"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long,
                                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
     ("recurrent", "fx_gated_head_norm"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p,
                                           c_long, c_int, c_int, c_int, c_float],
@@ -749,7 +749,8 @@ def short_conv(x, taps, state, token_seq, seq_starts, slot_ids, n_seqs: int) -> 
 
 def delta_prepare(q, k, a, b, A_log, dt_bias, n_heads: int, n_kv_heads: int, key_dim: int):
     """From convolved q, k [T, G*D], the decay's projection a [T, H*D] and the step size's b [T, H] (float32 rows):
-    (q / |q| / sqrt(D), k / |k|, exp(-exp(A_log[h]) softplus(a + dt_bias)), sigmoid(b)), all float32 contiguous."""
+    (q / |q| / sqrt(D), k / |k|, exp(-exp(A_log[h]) softplus(a + dt_bias)), sigmoid(b), the normed k . q per q/k head
+    [T, G]), all float32 contiguous."""
     T = q.shape[0]
     H, G, D = int(n_heads), int(n_kv_heads), int(key_dim)
     _f32_rows(q, "delta_prepare: q", G * D), _f32_rows(k, "delta_prepare: k", G * D)
@@ -762,19 +763,20 @@ def delta_prepare(q, k, a, b, A_log, dt_bias, n_heads: int, n_kv_heads: int, key
     kn = torch.empty((T, G * D), dtype=torch.float32, device=dev)
     decay = torch.empty((T, H * D), dtype=torch.float32, device=dev)
     beta = torch.empty((T, H), dtype=torch.float32, device=dev)
+    kq = torch.empty((T, G), dtype=torch.float32, device=dev)
     _call("recurrent", "fx_delta_prepare", _stream(), _p(q), q.stride(0), _p(k), k.stride(0), _p(a), a.stride(0), _p(b),
-          b.stride(0), _p(A_log), _p(dt_bias), dtype_code(A_log.dtype), _p(qn), _p(kn), _p(decay), _p(beta), T, H, G, D)
-    return qn, kn, decay, beta
+          b.stride(0), _p(A_log), _p(dt_bias), dtype_code(A_log.dtype), _p(qn), _p(kn), _p(decay), _p(beta), _p(kq), T, H, G, D)
+    return qn, kn, decay, beta, kq
 
 
-def channel_delta(qn, kn, decay, beta, v, state, seq_starts, slot_ids, n_seqs: int, n_heads: int, n_kv_heads: int,
+def channel_delta(qn, kn, decay, beta, kq, v, state, seq_starts, slot_ids, n_seqs: int, n_heads: int, n_kv_heads: int,
                   key_dim: int, v_dim: int) -> torch.Tensor:
     """The gated delta rule with a decay per key channel, over each sequence's tokens in order, from and into
     state[slot] (float32 [slots, H, V, D], the state's transpose: a column's key channels lie together):  S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;
-    o_t = S^T q_t.  Returns o float32 [T, H*V]."""
+    o_t = S^T q_t.  qn, kn, decay, beta, kq are what `delta_prepare` returns.  Returns o float32 [T, H*V]."""
     T = qn.shape[0]
     H, G, D, V = int(n_heads), int(n_kv_heads), int(key_dim), int(v_dim)
-    for t, cols, what in ((qn, G * D, "q"), (kn, G * D, "k"), (decay, H * D, "decay"), (beta, H, "beta")):
+    for t, cols, what in ((qn, G * D, "q"), (kn, G * D, "k"), (decay, H * D, "decay"), (beta, H, "beta"), (kq, G, "k.q")):
         if t.dtype != torch.float32 or not t.is_contiguous() or tuple(t.shape) != (T, cols):
             raise KernelError(f"channel_delta: {what} must be contiguous float32 [{T}, {cols}]")
     _f32_rows(v, "channel_delta: v", H * V)
@@ -783,7 +785,7 @@ def channel_delta(qn, kn, decay, beta, v, state, seq_starts, slot_ids, n_seqs: i
     if seq_starts.numel() < n_seqs + 1 or slot_ids.numel() < n_seqs:
         raise KernelError("channel_delta: the step's index tensors are shorter than its sequences")
     out = torch.empty((T, H * V), dtype=torch.float32, device=qn.device)
-    _call("recurrent", "fx_channel_delta", _stream(), _p(qn), _p(kn), _p(decay), _p(beta), _p(v), v.stride(0), _p(out),
+    _call("recurrent", "fx_channel_delta", _stream(), _p(qn), _p(kn), _p(decay), _p(beta), _p(kq), _p(v), v.stride(0), _p(out),
           out.stride(0), _p(state), _p(_i32(seq_starts, "seq_starts")), _p(_i32(slot_ids, "slot_ids")), int(n_seqs), H, G, D, V)
     return out
 

@@ -104,10 +104,10 @@ class ChannelDelta(Mixer):
         debug.region("delta gates")
         a = ops.gemm(proj[:, o1:o2], self.decay_out, epilogue=ops.EPI_STORE_F32)
         gate = ops.gemm(proj[:, o2:o2 + self.gate_rank], self.gate_out, epilogue=ops.EPI_STORE_F32)
-        qn, kn, decay, beta = ops.delta_prepare(conv[:, :QK], conv[:, QK:2 * QK], a, proj[:, C:o1], self.A_log, self.dt_bias,
+        qn, kn, decay, beta, kq = ops.delta_prepare(conv[:, :QK], conv[:, QK:2 * QK], a, proj[:, C:o1], self.A_log, self.dt_bias,
                                                 H, G, D)
         debug.region("delta rule")
-        o = ops.channel_delta(qn, kn, decay, beta, conv[:, 2 * QK:], cache.state["S"], starts, ctx.slot_ids, ctx.n_seqs,
+        o = ops.channel_delta(qn, kn, decay, beta, kq, conv[:, 2 * QK:], cache.state["S"], starts, ctx.slot_ids, ctx.n_seqs,
                               H, G, D, V)
         debug.region("delta out")
         y = ops.gated_head_norm(o, gate, self.norm_w, self.norm_eps, H, V, ctx.act_dtype)
