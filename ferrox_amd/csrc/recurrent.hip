@@ -13,26 +13,58 @@ FX_DEFINE_LAST_ERROR()
 //   y[t, c] = silu(sum_j taps[c, n-1-j] * x[t-j, c]),   j < n
 // where x[t-j] is a token of this step if it lies in the sequence's portion, else one of the n-1
 // inputs carried from before the portion (state[slot, c, :], oldest first; zeros at a sequence's start).
-// One thread per (token, channel).
+// One thread per (four tokens that follow each other in the batch, channel).
 // ---------------------------------------------------------------------------
 #define CONV_MAX_TAPS 16
+#define CONV_TOKENS 4        // tokens to a thread: neighbouring tokens share all but one of their inputs
+template <int TAPS>          // the number of taps where it is 2..4 (the inputs then live in registers), else 0
 __global__ __launch_bounds__(256) void short_conv_kernel(const float* __restrict__ x, long ldx, float* __restrict__ y, long ldy,
                                                          const void* __restrict__ taps, int taps_dtype, int n_taps,
                                                          const float* __restrict__ state, const int* __restrict__ token_seq,
                                                          const int* __restrict__ seq_starts, const int* __restrict__ slots,
-                                                         int C) {
-    const int t = blockIdx.y;
+                                                         int n_tokens, int C) {
+    const int t0 = blockIdx.y * CONV_TOKENS;
     const int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
-    const int s = token_seq[t];
-    const int i = t - seq_starts[s];                 // place in the portion
-    const float* carried = state + ((size_t)slots[s] * C + c) * (n_taps - 1);
-    float acc = 0.f;
-    for (int j = n_taps - 1; j >= 0; --j) {          // oldest input first
-        const float xv = j <= i ? x[(size_t)(t - j) * ldx + c] : carried[n_taps - 1 + i - j];
-        acc = fmaf(load_as_float(taps, taps_dtype, (size_t)c * n_taps + n_taps - 1 - j), xv, acc);
+    if constexpr (TAPS > 0) {
+        // the inputs of tokens t0 - TAPS + 1 .. t0 + 3 once, then every token of the four takes its own from them (those
+        // of its sequence's portion) or from what its sequence carried
+        float w[TAPS], xin[CONV_TOKENS + TAPS - 1];
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) w[j] = load_as_float(taps, taps_dtype, (size_t)c * TAPS + j);
+#pragma unroll
+        for (int e = 0; e < CONV_TOKENS + TAPS - 1; ++e) {
+            const int t = t0 - (TAPS - 1) + e;
+            xin[e] = (t >= 0 && t < n_tokens) ? x[(size_t)t * ldx + c] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < CONV_TOKENS; ++u) {
+            const int t = t0 + u;
+            if (t >= n_tokens) break;
+            const int s = token_seq[t];
+            const int i = t - seq_starts[s];             // place in the portion
+            const float* carried = state + ((size_t)slots[s] * C + c) * (TAPS - 1);
+            float acc = 0.f;
+#pragma unroll
+            for (int j = TAPS - 1; j >= 0; --j) {        // oldest input first
+                const float xv = j <= i ? xin[u + TAPS - 1 - j] : carried[TAPS - 1 + i - j];
+                acc = fmaf(w[TAPS - 1 - j], xv, acc);
+            }
+            y[(size_t)t * ldy + c] = acc / (1.0f + expf(-acc));
+        }
+    } else {
+        for (int t = t0; t < min(t0 + CONV_TOKENS, n_tokens); ++t) {
+            const int s = token_seq[t];
+            const int i = t - seq_starts[s];
+            const float* carried = state + ((size_t)slots[s] * C + c) * (n_taps - 1);
+            float acc = 0.f;
+            for (int j = n_taps - 1; j >= 0; --j) {
+                const float xv = j <= i ? x[(size_t)(t - j) * ldx + c] : carried[n_taps - 1 + i - j];
+                acc = fmaf(load_as_float(taps, taps_dtype, (size_t)c * n_taps + n_taps - 1 - j), xv, acc);
+            }
+            y[(size_t)t * ldy + c] = acc / (1.0f + expf(-acc));
+        }
     }
-    y[(size_t)t * ldy + c] = acc / (1.0f + expf(-acc));
 }
 
 // After the step: the last n-1 inputs of every sequence, oldest first.  One thread per (sequence, channel);
@@ -59,12 +91,17 @@ FX_API int fx_short_conv(void* stream, const float* x, long ldx, float* y, long 
     FX_REQUIRE(n_taps >= 1 && n_taps <= CONV_MAX_TAPS, "short_conv: %d taps, this kernel takes 1..%d", n_taps, CONV_MAX_TAPS);
     FX_REQUIRE(ldx >= C && ldy >= C, "short_conv: rows of %ld and %ld hold fewer than %d channels", ldx, ldy, C);
     FX_REQUIRE(taps_dtype == FX_F32 || taps_dtype == FX_BF16, "short_conv: unknown dtype %d of the taps", taps_dtype);
-    FX_REQUIRE(T <= 65535 && n_seqs <= 65535, "short_conv: %d tokens of %d sequences are more than a launch takes", T, n_seqs);
+    FX_REQUIRE(T <= 4 * 65535 && n_seqs <= 65535, "short_conv: %d tokens of %d sequences are more than a launch takes", T, n_seqs);
     FX_REQUIRE(x != y, "short_conv: the output must not be the input (carried inputs are read from it afterwards)");
     if (T == 0 || n_seqs == 0) return 0;
     hipStream_t s = (hipStream_t)stream;
-    short_conv_kernel<<<dim3((C + 255) / 256, T), 256, 0, s>>>(x, ldx, y, ldy, taps, taps_dtype, n_taps, state, token_seq,
-                                                               seq_starts, slots, C);
+    const dim3 grid((C + 255) / 256, (T + CONV_TOKENS - 1) / CONV_TOKENS);
+#define FX_CONV(TAPS_) short_conv_kernel<TAPS_><<<grid, 256, 0, s>>>(x, ldx, y, ldy, taps, taps_dtype, n_taps, state, token_seq, seq_starts, slots, T, C)
+    if (n_taps == 4) FX_CONV(4);
+    else if (n_taps == 3) FX_CONV(3);
+    else if (n_taps == 2) FX_CONV(2);
+    else FX_CONV(0);
+#undef FX_CONV
     if (n_taps > 1)
         conv_carry_kernel<<<dim3((C + 255) / 256, n_seqs), 256, 0, s>>>(x, ldx, state, seq_starts, slots, C, n_taps);
     FX_CHECK_LAUNCH("short_conv");
