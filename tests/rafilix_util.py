@@ -49,9 +49,9 @@ CFG_MAIN = config([
 ], width=64, vocab=160)
 # bfloat16 on the matrix units: equal head sizes that are multiples of 16, widths that are multiples of 64
 CFG_MFMA = config([
-    attention_layer(heads=4, kv_heads=2, dim=64, vdim=64, chunk=40, rot_dims=64, scaling=(8.0, 1.0, 4.0, 96.0), scale=0.3,
-                    mlp=moe(6, 2, 2, 64)),
-    delta_layer(heads=4, kv_heads=4, dim=64, vdim=32, conv=4, mlp=moe(6, 2, 2, 64)),
+    attention_layer(heads=4, kv_heads=2, dim=64, vdim=64, chunk=40, rot_dims=64, scaling=(4.0, 1.0, 8.0, 96.0), scale=0.3,
+                    mlp=moe(6, 1, 3, 64)),
+    delta_layer(heads=4, kv_heads=4, dim=64, vdim=48, conv=3, mlp=moe(5, 3, 2, 64)),
     attention_layer(heads=2, kv_heads=2, dim=32, vdim=32, chunk=100, rot_dims=32, scale=0.4, mlp=None),
 ], width=128, vocab=256)
 
