@@ -170,6 +170,50 @@ FX_API int fx_delta_prepare(void* stream, const float* q, long ldq, const float*
 }
 
 // ---------------------------------------------------------------------------
+// Two small float32 products of few rows in one launch: out_i[t, n] = sum_k x_i[t, k] * wt_i[k, n], i = 0, 1, k
+// ascending in one accumulator (the sums of the float32 product kernel, so a row gets the same bits from either).
+// These are the second halves of the delta rule's two low-rank projections (decay and output gate): K is the
+// inner size (tens to a few hundred), the weights are kept transposed [K, N] so that neighbouring lanes read
+// neighbouring columns, and a decode step's few rows make them two launches' worth of waiting otherwise.
+// Grid: (ceil(max N / 256), rows, 2).
+// ---------------------------------------------------------------------------
+#define PAIR_MAX_K 512
+__global__ __launch_bounds__(256) void small_rows_pair_kernel(const float* __restrict__ x0, long ldx0, const float* __restrict__ wt0,
+                                                              float* __restrict__ out0, long ldo0, int K0, int N0,
+                                                              const float* __restrict__ x1, long ldx1, const float* __restrict__ wt1,
+                                                              float* __restrict__ out1, long ldo1, int K1, int N1) {
+    __shared__ float xs[PAIR_MAX_K];
+    const bool second = blockIdx.z == 1;
+    const float* x = second ? x1 : x0;
+    const float* wt = second ? wt1 : wt0;
+    float* out = second ? out1 : out0;
+    const long ldx = second ? ldx1 : ldx0, ldo = second ? ldo1 : ldo0;
+    const int K = second ? K1 : K0, N = second ? N1 : N0;
+    const int t = blockIdx.y, n = blockIdx.x * 256 + threadIdx.x;
+    if (blockIdx.x * 256 >= N) return;               // (the same in every thread of the block)
+    for (int k = threadIdx.x; k < K; k += 256) xs[k] = x[(size_t)t * ldx + k];
+    __syncthreads();
+    if (n >= N) return;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int k = 0; k < K; ++k) acc = fmaf(xs[k], wt[(size_t)k * N + n], acc);
+    out[(size_t)t * ldo + n] = acc;
+}
+
+FX_API int fx_small_rows_pair(void* stream, const float* x0, long ldx0, const float* wt0, float* out0, long ldo0, int K0, int N0,
+                              const float* x1, long ldx1, const float* wt1, float* out1, long ldo1, int K1, int N1, int T) {
+    FX_REQUIRE(T >= 0 && T <= 65535, "small_rows_pair: %d rows", T);
+    FX_REQUIRE(K0 >= 1 && K0 <= PAIR_MAX_K && K1 >= 1 && K1 <= PAIR_MAX_K, "small_rows_pair: inner sizes %d and %d, this kernel takes 1..%d", K0, K1, PAIR_MAX_K);
+    FX_REQUIRE(N0 >= 1 && N1 >= 1 && ldx0 >= K0 && ldx1 >= K1 && ldo0 >= N0 && ldo1 >= N1, "small_rows_pair: bad sizes");
+    if (T == 0) return 0;
+    const int widest = N0 > N1 ? N0 : N1;
+    small_rows_pair_kernel<<<dim3((widest + 255) / 256, T, 2), 256, 0, (hipStream_t)stream>>>(x0, ldx0, wt0, out0, ldo0, K0, N0,
+                                                                                               x1, ldx1, wt1, out1, ldo1, K1, N1);
+    FX_CHECK_LAUNCH("small_rows_pair");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
 // The recurrence.  Per head, with S [D, V] carried from token to token:
 //   S <- diag(decay_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
 // Tokens follow each other; columns of S never meet.  A wave owns 64 / LPC columns, LPC = 16 or 32 lanes to a

@@ -74,6 +74,8 @@ _sigs = {
                                         c_int, c_int, c_int, c_int],
     ("recurrent", "fx_channel_delta"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_long,
                                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
+    ("recurrent", "fx_small_rows_pair"): [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int,
+                                          c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int],
     ("recurrent", "fx_gated_head_norm"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p,
                                           c_long, c_int, c_int, c_int, c_float],
     ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
@@ -802,3 +804,24 @@ def gated_head_norm(o, gate, weight, eps: float, n_heads: int, v_dim: int, out_d
     _call("recurrent", "fx_gated_head_norm", _stream(), dtype_code(out_dtype), _p(o), o.stride(0), _p(gate), gate.stride(0),
           _p(weight), dtype_code(weight.dtype), _p(y), y.stride(0), T, H, V, float(eps))
     return y
+
+
+SMALL_ROWS_MAX = 32          # up to so many rows the pair of small float32 products is one launch (more rows: the tiled product)
+SMALL_ROWS_MAX_K = 512
+
+
+def small_rows_pair(x0, wt0, x1, wt1):
+    """(x0 @ wt0, x1 @ wt1) in float32 for few rows, one launch: x_i float32 rows [T, K_i] (any row stride),
+    wt_i contiguous float32 [K_i, N_i] (the weights transposed).  The sums run over k ascending in one accumulator,
+    as `gemm` does in float32."""
+    T = x0.shape[0]
+    for x, wt in ((x0, wt0), (x1, wt1)):
+        _f32_rows(x, "small_rows_pair: x", wt.shape[0])
+        if wt.dtype != torch.float32 or wt.dim() != 2 or not wt.is_contiguous() or x.shape[1] != wt.shape[0] \
+                or wt.shape[0] > SMALL_ROWS_MAX_K or x.shape[0] != T:
+            raise KernelError(f"small_rows_pair: rows {tuple(x.shape)} against transposed weights {tuple(wt.shape)}")
+    out0 = torch.empty((T, wt0.shape[1]), dtype=torch.float32, device=x0.device)
+    out1 = torch.empty((T, wt1.shape[1]), dtype=torch.float32, device=x0.device)
+    _call("recurrent", "fx_small_rows_pair", _stream(), _p(x0), x0.stride(0), _p(wt0), _p(out0), out0.stride(0), wt0.shape[0],
+          wt0.shape[1], _p(x1), x1.stride(0), _p(wt1), _p(out1), out1.stride(0), wt1.shape[0], wt1.shape[1], T)
+    return out0, out1

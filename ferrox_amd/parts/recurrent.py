@@ -58,7 +58,7 @@ class ChannelDelta(Mixer):
         self.names = dict(self.TENSORS, **(names or {}))
         self.qk_width, self.v_width = self.n_kv_heads * self.key_dim, self.n_heads * self.v_dim
         self.conv_channels = 2 * self.qk_width + self.v_width
-        self.w_in = self.taps = self.decay_out = self.gate_out = self.A_log = self.dt_bias = self.norm_w = self.o_proj = None
+        self.w_in = self.taps = self.decay_out = self.gate_out = self.decay_out_t = self.gate_out_t = self.A_log = self.dt_bias = self.norm_w = self.o_proj = None
 
     def param_specs(self):
         W, n = self.hidden_size, self.names
@@ -82,6 +82,8 @@ class ChannelDelta(Mixer):
         self.taps = torch.cat([fetch(n[x]).float() for x in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
         self.decay_out = fetch(n["decay_out"]).float().contiguous()
         self.gate_out = fetch(n["gate_out"]).float().contiguous()
+        # (transposed copies for the few rows of a decode step, where both products are one launch)
+        self.decay_out_t, self.gate_out_t = self.decay_out.t().contiguous(), self.gate_out.t().contiguous()
         self.A_log = fetch(n["A_log"]).float().contiguous()
         self.dt_bias = fetch(n["dt_bias"]).float().contiguous()
         self.norm_w = fetch(n["norm"]).contiguous()
@@ -102,8 +104,11 @@ class ChannelDelta(Mixer):
         debug.region("delta conv")
         conv = ops.short_conv(proj[:, :C], self.taps, cache.state["conv"], ctx.token_seq, starts, ctx.slot_ids, ctx.n_seqs)
         debug.region("delta gates")
-        a = ops.gemm(proj[:, o1:o2], self.decay_out, epilogue=ops.EPI_STORE_F32)
-        gate = ops.gemm(proj[:, o2:o2 + self.gate_rank], self.gate_out, epilogue=ops.EPI_STORE_F32)
+        if ctx.n_tokens <= ops.SMALL_ROWS_MAX and max(self.decay_rank, self.gate_rank) <= ops.SMALL_ROWS_MAX_K:
+            a, gate = ops.small_rows_pair(proj[:, o1:o2], self.decay_out_t, proj[:, o2:o2 + self.gate_rank], self.gate_out_t)
+        else:
+            a = ops.gemm(proj[:, o1:o2], self.decay_out, epilogue=ops.EPI_STORE_F32)
+            gate = ops.gemm(proj[:, o2:o2 + self.gate_rank], self.gate_out, epilogue=ops.EPI_STORE_F32)
         qn, kn, decay, beta, kq = ops.delta_prepare(conv[:, :QK], conv[:, QK:2 * QK], a, proj[:, C:o1], self.A_log, self.dt_bias,
                                                 H, G, D)
         debug.region("delta rule")

@@ -124,6 +124,22 @@ def test_stored_activation_of_the_product():
         assert torch.allclose(got.double(), want, atol=1e-5 if dt == torch.float32 else 3e-2, rtol=1e-2)
 
 
+def test_pair_of_small_products():
+    """The one-launch pair of float32 products for few rows against float64 products, and bit for bit against the
+    float32 product kernel that takes more rows (a row must not change with the number of rows beside it)."""
+    from ferrox_amd import ops
+    gen = torch.Generator().manual_seed(8)
+    for T, K0, N0, K1, N1 in ((1, 12, 40, 20, 7), (9, 128, 600, 64, 300), (32, 5, 3, 300, 257)):
+        big = torch.randn(T, K0 + K1 + 3, generator=gen).cuda()
+        x0, x1 = big[:, :K0], big[:, K0 + 3:]                       # rows with a stride of their own
+        w0, w1 = torch.randn(N0, K0, generator=gen).cuda(), torch.randn(N1, K1, generator=gen).cuda()
+        a, b = ops.small_rows_pair(x0, w0.t().contiguous(), x1, w1.t().contiguous())
+        for got, x, w in ((a, x0, w0), (b, x1, w1)):
+            want = x.double() @ w.double().T
+            assert torch.allclose(got.double(), want, atol=1e-4 * float(want.abs().max()))
+            assert torch.equal(got, ops.gemm(x, w, epilogue=ops.EPI_STORE_F32))
+
+
 # ---------------------------------------------------------------------------
 # the model whole and cut
 # ---------------------------------------------------------------------------
