@@ -127,7 +127,9 @@ def main(argv=None) -> int:
         if args.random_weights:
             from .config.base import read_config_json
             raw = read_config_json(args.config) if os.path.exists(args.config) else presets.load(args.config)
-            if args.layers > 0:
+            if args.layers > 0 and isinstance(raw.get("layers"), list):      # a design that lists its layers: the first N, repeated if short
+                raw = dict(raw, layers=[raw["layers"][i % len(raw["layers"])] for i in range(args.layers)])
+            elif args.layers > 0:
                 raw = dict(raw, num_hidden_layers=args.layers)
             source = dict(config=raw, random_weights=seed)
             print(f"random weights: seed {seed}, configuration {args.config}", file=sys.stderr)

@@ -344,3 +344,9 @@ def test_command_line_generates(tmp_path_factory):
                          capture_output=True, text=True, timeout=300)
     assert out.returncode == 0, out.stderr[-2000:]
     assert ",".join(map(str, want)) in out.stdout.replace(" ", ""), (out.stdout[-500:], want)
+    # without a folder: random weights of a named shape of the design (two of its layers)
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "ferrox-amd"), "--random-weights", "--config", "rafilix-2k",
+                          "--layers", "2", "-s", "5", "--tokens", "1,2,3", "-n", "4", "--temp", "0", "--ignore-eos",
+                          "--num-pages", "8"], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    assert len(out.stdout.strip().split(",")) == 4, out.stdout[-300:]

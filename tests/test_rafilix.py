@@ -136,6 +136,16 @@ def test_config_reads_every_layer_and_refuses_what_it_does_not_know():
         assert word in str(e.value), (word, str(e.value))
 
 
+def test_named_shape_of_the_design_reads():
+    from ferrox_amd.config import presets
+    from ferrox_amd.models.registry import resolve
+    raw = presets.load("rafilix-2k")
+    assert resolve(raw).name == "Rafilix"
+    cfg = RafilixConfig.from_dict(raw)
+    assert len(cfg.layers) == 8 and {l.type for l in cfg.layers} == {"attention", "channel_delta"}
+    assert cfg.layers[1].mixer.decay_rank == cfg.layers[1].mixer.dim        # named in the file: no checkpoint gives it
+
+
 def test_description_names_the_tensors_of_the_test_models():
     """The tensor names and shapes that the model description expects are those that the tests' own list gives
     (written from the design, not from the description); the low-rank sizes come from the tensors."""
