@@ -49,6 +49,8 @@ def _native():
             fn = getattr(lib, "fxc_" + name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.c_void_p, ctypes.c_int64] + extra
+        lib.fxc_keep_first.restype = ctypes.c_int
+        lib.fxc_keep_first.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
         lib.fxc_release.restype = None
         lib.fxc_release.argtypes = [ctypes.c_void_p, ctypes.c_int64]
         for name, extra in (("n_free_pages", [ctypes.c_int]), ("num_pages", [ctypes.c_int]), ("n_free_slots", []),
@@ -69,16 +71,25 @@ def _native():
 
 def _window_code(window) -> int:
     """How a group's pages age, as the native manager numbers it: None keeps every position (-1), an int W keeps the
-    last W, ("chunk", C) keeps the positions of the chunk of C that the sequence's end lies in (-(C + 1))."""
+    last W, ("chunk", C) keeps the positions of the chunk of C that the sequence's end lies in (-(C + 1)),
+    ("keep", W, F) keeps the last W like W alone (the first F are the business of `_kept_first`)."""
     if window is None:
         return -1
     if isinstance(window, tuple):
+        if len(window) == 3 and window[0] == "keep" and int(window[1]) >= 1 and int(window[2]) >= 0:
+            return int(window[1])
         if len(window) != 2 or window[0] != "chunk" or int(window[1]) < 1:
-            raise ValueError(f"a group's window is None, a number of positions or ('chunk', size), not {window!r}")
+            raise ValueError(f"a group's window is None, a number of positions, ('chunk', size) or "
+                             f"('keep', window, first), not {window!r}")
         return -(int(window[1]) + 1)
     if int(window) < 0:
         raise ValueError(f"a window of {window} positions")
     return int(window)
+
+
+def _kept_first(window) -> int:
+    """The number of first positions of a sequence whose pages a windowed group never gives back."""
+    return int(window[2]) if isinstance(window, tuple) and window[0] == "keep" else 0
 
 
 class _Core:
@@ -97,6 +108,9 @@ class _Core:
         self.h = self.lib.fxc_create(n, w, p, block_size, n_slots)
         if not self.h:
             raise ValueError("the cache manager refused its sizes")
+        for g, x in enumerate(windows):
+            if _kept_first(x) and self.lib.fxc_keep_first(self.h, g, _kept_first(x)) != 0:
+                raise ValueError(self.error())
 
     def __del__(self):
         h, self.h = getattr(self, "h", None), None

@@ -5,7 +5,10 @@
 // [n_seqs, max_blocks].  A query at position p sees key t iff t <= p and, with a
 // window W > 0, p - t < W (ferrox-core/src/attention.rs:441-447, 498-513), or, with a
 // chunked mask of C > 0 positions, t >= floor(p / C) * C (chunks count from position 0
-// of the sequence).  A value head may have another size (vd) than a query and key
+// of the sequence).  With a window, the first `keep_first` keys of a sequence may stay visible to
+// every later query (t < keep_first), and a head may have a sink: one more term exp(sink_h) in the
+// softmax's denominator, with no key and no value.  The output may be gated: out * sigmoid(gate),
+// gate a matrix of out's shape.  A value head may have another size (vd) than a query and key
 // head (hd); the bfloat16 MFMA kernels take equal sizes, the others both.  Head
 // h reads kv head h / (n_heads / n_kv_heads) (attention.rs:432-438).  Scores,
 // softmax and the output sum are float32, in the one-pass form of
@@ -36,6 +39,10 @@ struct AttnArgs {
     int nh, nkv, hd, bs, window;
     int vd;              // size of a value head (and of an output head)
     int mask_chunk;      // > 0: the chunked mask
+    int keep_first;      // > 0 (with a window): keys t < keep_first stay visible to every later query
+    const float* sinks;  // [n_heads] or null: a logit per head that joins the softmax's denominator
+    const void* gate;    // [tokens, n_heads * vd] or null (type of out): the output is multiplied by sigmoid(gate)
+    long ldg;
     int bs_shift;        // log2(bs) if bs is a power of two, else -1
     int n_items;
     float scale;
@@ -59,6 +66,52 @@ __device__ __forceinline__ int first_visible(const AttnArgs& a, int p) {
 }
 // whether queries see a bounded stretch of keys (a window or a chunk) rather than all before them
 __device__ __forceinline__ bool bounded_keys(const AttnArgs& a) { return a.window > 0 || a.mask_chunk > 0; }
+
+// The keys a block may touch: t < end and (t >= begin or t < keep), keep being the kept first keys of the
+// sequence (0: none).  Pages of other keys may have been given back.
+struct KeySpan {
+    int begin, end, keep;
+    __device__ __forceinline__ bool has(int t) const { return t < end && (t >= begin || t < keep); }
+    // whether any of the n consecutive keys from t on is one of them
+    __device__ __forceinline__ bool touches(int t, int n) const { return t < end && (t + n > begin || t < keep); }
+    // whether all of the 64 keys of the tile at t are
+    __device__ __forceinline__ bool holds_tile(int t) const { return t >= begin && t + 64 <= end; }
+};
+// The tiles of 64 keys that a block walks over, in ascending order: those that hold kept first keys and lie
+// before the first tile of the span's stretch [begin, end), then that stretch's tiles.
+struct TileWalk {
+    int n_keep, first, n;
+    __device__ __forceinline__ int start(int i) const { return i < n_keep ? 64 * i : first + 64 * (i - n_keep); }
+};
+__device__ __forceinline__ TileWalk tile_walk(const KeySpan& k) {
+    TileWalk w;
+    w.first = k.begin & ~63;
+    w.n_keep = min((k.keep + 63) >> 6, w.first >> 6);
+    w.n = w.n_keep + max(0, (k.end - w.first + 63) >> 6);
+    return w;
+}
+
+// What a row's running maximum m and sum l become when the head's sink joins the denominator: the factor
+// for the row's output, already divided by the new sum.  `m` and `sink` in the same units (natural logarithm,
+// or base 2 where the caller's maximum is).
+template <bool BASE2>
+__device__ __forceinline__ float finish_row(const AttnArgs& a, int h, float m, float l) {
+    if (!a.sinks) return 1.f / l;
+    const float sk = BASE2 ? a.sinks[h] * 1.4426950408889634f : a.sinks[h];
+    const float top = fmaxf(m, sk);      // (m is finite: a query sees itself)
+    const float f = BASE2 ? __builtin_amdgcn_exp2f(m - top) : expf(m - top);
+    const float e = BASE2 ? __builtin_amdgcn_exp2f(sk - top) : expf(sk - top);
+    return f / (l * f + e);
+}
+// one output element on its way out: through the gate, if there is one
+template <typename T>
+__device__ __forceinline__ void store_out(const AttnArgs& a, int tok, int h, int d, float v) {
+    if (a.gate) {
+        const float gv = to_float(((const T*)a.gate)[(size_t)tok * a.ldg + (size_t)h * a.vd + d]);
+        v *= 1.f / (1.f + expf(-gv));
+    }
+    from_float((T*)a.out + (size_t)tok * a.ldo + (size_t)h * a.vd + d, v);
+}
 
 // block of the table and slot in its page of key t (a shift when the page size is a power of two)
 __device__ __forceinline__ void page_slot(const AttnArgs& a, int t, int& blk, int& slot) {
@@ -133,6 +186,8 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
     const int pmin = a.positions[tok0], pmax = a.positions[tok0 + n - 1];
     const int kv_begin = first_visible(a, pmin);
     const int kv_end = pmax + 1;
+    const KeySpan span = {kv_begin, kv_end, a.keep_first};
+    const TileWalk walk = tile_walk(span);
 
     float m[TQ], l[TQ], o[HD_MAX / 64][TQ];
 #pragma unroll
@@ -144,9 +199,10 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
     }
     __syncthreads();
 
-    for (int kt0 = (kv_begin / 64) * 64; kt0 < kv_end; kt0 += 64) {
+    for (int ti = 0; ti < walk.n; ++ti) {
+        const int kt0 = walk.start(ti);
         const int t = kt0 + lane;
-        const bool in_range = t >= kv_begin && t < kv_end;
+        const bool in_range = span.has(t);
         float s[TQ];
 #pragma unroll
         for (int i = 0; i < TQ; ++i) s[i] = 0.f;
@@ -161,7 +217,7 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
         float al[TQ];
 #pragma unroll
         for (int i = 0; i < TQ; ++i) {
-            const bool vis = in_range && t <= pos[i] && t >= first_visible(a, pos[i]);
+            const bool vis = in_range && t <= pos[i] && (t >= first_visible(a, pos[i]) || t < a.keep_first);
             const float sv = vis ? s[i] : NEG_INF;
             const float m_new = fmaxf(m[i], wave_max(sv));
             al[i] = (m_new == NEG_INF) ? 1.f : expf(m[i] - m_new);
@@ -178,7 +234,8 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
 #pragma unroll
                 for (int i = 0; i < TQ; ++i) o[dd][i] *= al[i];
                 const int jn = min(64, kv_end - kt0);
-                for (int j = max(0, kv_begin - kt0); j < jn; ++j) {
+                for (int j = 0; j < jn; ++j) {
+                    if (!span.has(kt0 + j)) continue;
                     const float vv = to_float(value_col<T>(a, bt, kvh, kt0 + j)[(size_t)d * a.bs]);
 #pragma unroll
                     for (int i = 0; i < TQ; ++i) o[dd][i] = fmaf(Ps[i][j], vv, o[dd][i]);
@@ -193,8 +250,7 @@ __global__ __launch_bounds__(64) void attn_tile_kernel(AttnArgs a) {
         if (d < a.vd) {
 #pragma unroll
             for (int i = 0; i < TQ; ++i)
-                if (i < n)
-                    from_float((T*)a.out + (size_t)(tok0 + i) * a.ldo + (size_t)h * a.vd + d, o[dd][i] / l[i]);
+                if (i < n) store_out<T>(a, tok0 + i, h, d, o[dd][i] * finish_row<false>(a, h, m[i], l[i]));
         }
     }
 }
@@ -214,11 +270,14 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
     const int* bt = a.block_table + (size_t)a.item_seq[item] * a.max_blocks;
     const int hd = a.hd;
     const int p = a.positions[tok];
-    const int kv_begin = max(first_visible(a, p), split * a.chunk);
-    const int kv_end = min(p + 1, (split + 1) * a.chunk);
+    // the split's keys [split * chunk, (split + 1) * chunk) of which the query sees those from its window's first
+    // on and the kept first ones
+    const int s0 = split * a.chunk;
+    const KeySpan span = {max(first_visible(a, p), s0), min(p + 1, s0 + a.chunk), a.keep_first};
+    const int kv_end = span.end;
     float* po = a.part_o + (((size_t)item * a.nh + h) * a.splits + split) * a.vd;
     float* pml = a.part_ml + (((size_t)item * a.nh + h) * a.splits + split) * 2;
-    if (kv_begin >= kv_end) {
+    if (s0 >= kv_end || !(span.begin < kv_end || s0 < span.keep)) {
         if (lane == 0) {
             pml[0] = NEG_INF;
             pml[1] = 0.f;
@@ -230,9 +289,10 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
     float m = NEG_INF, l = 0.f, o[HD_MAX / 64];
 #pragma unroll
     for (int dd = 0; dd < HD_MAX / 64; ++dd) o[dd] = 0.f;
-    for (int kt0 = (kv_begin / 64) * 64; kt0 < kv_end; kt0 += 64) {
+    for (int kt0 = s0; kt0 < kv_end; kt0 += 64) {
+        if (!span.touches(kt0, 64)) continue;      // a tile between the kept keys and the window
         const int t = kt0 + lane;
-        const bool vis = t >= kv_begin && t < kv_end;
+        const bool vis = span.has(t);
         float s = 0.f;
         if (vis) {
             const T* kr = key_row<T>(a, bt, kvh, t);
@@ -240,7 +300,7 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
         }
         const float sv = vis ? s : NEG_INF;
         const float m_new = fmaxf(m, wave_max(sv));
-        const float al = expf(m - m_new);  // a tile inside [kv_begin, kv_end) always has a visible key
+        const float al = (m_new == NEG_INF) ? 1.f : expf(m - m_new);
         const float pr = vis ? expf(sv - m_new) : 0.f;
         l = l * al + wave_sum(pr);
         m = m_new;
@@ -252,8 +312,10 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(AttnArgs a) {
             if (d < a.vd) {
                 float acc = o[dd] * al;
                 const int jn = min(64, kv_end - kt0);
-                for (int j = max(0, kv_begin - kt0); j < jn; ++j)
+                for (int j = 0; j < jn; ++j) {
+                    if (!span.has(kt0 + j)) continue;
                     acc = fmaf(Ps[j], to_float(value_col<T>(a, bt, kvh, kt0 + j)[(size_t)d * a.bs]), acc);
+                }
                 o[dd] = acc;
             }
         }
@@ -301,6 +363,7 @@ __global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a) {
     __syncthreads();
     float l = 0.f;
     for (int s = 0; s < S; ++s) l += wsm[s] * ((wsm[s] > 0.f) ? pml[2 * s + 1] : 0.f);   // ascending, the same in every thread
+    const float fin = finish_row<false>(a, h, m, l);
     for (int d = tid; d < hd; d += 128) {
         float acc = 0.f;
         int s0 = 0;
@@ -318,7 +381,7 @@ __global__ __launch_bounds__(128) void attn_decode_merge_kernel(AttnArgs a) {
             const float v = (w > 0.f) ? po[(size_t)s * hd + d] : 0.f;   // an empty chunk wrote nothing
             acc = fmaf(w, v, acc);
         }
-        from_float((T*)a.out + (size_t)tok * a.ldo + (size_t)h * hd + d, acc / l);
+        store_out<T>(a, tok, h, d, acc * fin);
     }
 }
 
@@ -367,11 +430,11 @@ __device__ __forceinline__ float quad_sum(float x) {
 // One step of the one-pass softmax on a lane's 16 raw scores sc[kb][r] of keys key0 + 4*kb + r
 // (key0 = tile start + 16g), in base 2: t = score * c with c = scale * log2(e), m and l are the
 // running maximum (of t) and sum of this lane's row, shared by the row's four lanes.  MASKED: only
-// keys in [lo, hi] count.  Returns the factor for what was accumulated so far, and the
+// keys in [lo, hi] count, and those below `keep` that are no later than hi.  Returns the factor for what was accumulated so far, and the
 // probabilities rounded to bfloat16: p_lo for keys key0 .. key0+7, p_hi for key0+8 .. key0+15.
 template <bool MASKED>
 __device__ __forceinline__ float softmax_step(f32x4_t (&sc)[4], int key0, int lo, int hi, float c, float& m, float& l,
-                                              uint4& p_lo, uint4& p_hi) {
+                                              uint4& p_lo, uint4& p_hi, int keep = 0) {
     // the maximum is taken over the raw scores and scaled once (c > 0, and rounding keeps the order); a score's
     // exponent is then one fused multiply-add, score * c - maximum
     float mt = NEG_INF;
@@ -381,7 +444,7 @@ __device__ __forceinline__ float softmax_step(f32x4_t (&sc)[4], int key0, int lo
         for (int r = 0; r < 4; ++r) {
             if (MASKED) {
                 const int key = key0 + 4 * kb + r;
-                sc[kb][r] = (key >= lo && key <= hi) ? sc[kb][r] : NEG_INF;
+                sc[kb][r] = ((key >= lo || key < keep) && key <= hi) ? sc[kb][r] : NEG_INF;
             }
             mt = fmaxf(mt, sc[kb][r]);
         }
@@ -420,14 +483,14 @@ __device__ __forceinline__ f32x4_t pv_step(f32x4_t acc, bool rescale, const floa
     return acc;
 }
 
-// Eight consecutive keys' values (first_key ..): those outside [kv_begin, kv_end) become zeros.  Their
+// Eight consecutive keys' values (first_key ..): those outside the span become zeros.  Their
 // probabilities are zero, but what memory holds there need not be a number.
-__device__ __forceinline__ uint4 keep_keys(uint4 v, int first_key, int kv_begin, int kv_end) {
+__device__ __forceinline__ uint4 keep_keys(uint4 v, int first_key, const KeySpan& span) {
     uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const int key = first_key + e;
-        if (key < kv_begin || key >= kv_end) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
+        if (!span.has(key)) w[e >> 1] &= (e & 1) ? 0x0000ffffu : 0xffff0000u;
     }
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
@@ -465,9 +528,10 @@ struct WaveAttn {
         }
     }
 
-    // keys [kt0, kt0 + 64); this lane's row sees key t iff lo <= t <= hi (hi < lo: row unused)
-    __device__ __forceinline__ void tile(const AttnArgs& a, const PageLookup& pl, int kvh, int kt0, int kv_begin, int kv_end,
+    // keys [kt0, kt0 + 64); this lane's row sees key t iff t <= hi and (lo <= t or t < span.keep) (hi < lo: row unused)
+    __device__ __forceinline__ void tile(const AttnArgs& a, const PageLookup& pl, int kvh, int kt0, const KeySpan& span,
                                          int lo, int hi) {
+        const int kv_end = span.end;
         const int lane = threadIdx.x & 63, li = lane & 15, g = lane >> 4;
         const int l8 = li & 7, lh = li >> 3;
         const int hd = a.hd, bs = a.bs;
@@ -477,8 +541,8 @@ struct WaveAttn {
         // values first, so that they arrive while the scores are computed: 16 consecutive keys
         // kt0 + 16g .. of transposed row d = 16*cb + li
         const int kg = kt0 + 16 * g;
-        const bool edge = kt0 < kv_begin || kt0 + 64 > kv_end;      // some key of the tile is outside
-        const bool vlive = kg < kv_end && kg + 16 > kv_begin;
+        const bool edge = !span.holds_tile(kt0);      // some key of the tile is outside
+        const bool vlive = span.touches(kg, 16);
         const int vkey = vlive ? kg : safe_group;
         int vblk, vslot;
         page_slot(a, vkey, vblk, vslot);
@@ -492,7 +556,7 @@ struct WaveAttn {
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
             const int key0 = kt0 + 16 * (li >> 2) + 4 * kb + (li & 3);
-            klives[kb] = key0 >= kv_begin && key0 < kv_end;
+            klives[kb] = span.has(key0);
             int kblk;
             if (KP < KS) {
                 page_slot(a, klives[kb] ? key0 : safe_group, kblk, kslots[kb]);
@@ -500,9 +564,9 @@ struct WaveAttn {
             }
             // rows li % 8 and 8 + li % 8 of the block's 16 keys (row i is key 16 (i / 4) + 4 kb + i % 4 of the tile)
             const int key_a = kt0 + 16 * (l8 >> 2) + 4 * kb + (l8 & 3), key_b = key_a + 32;
-            page_slot(a, key_a >= kv_begin && key_a < kv_end ? key_a : safe_group, kblk, kslots_a[kb]);
+            page_slot(a, span.has(key_a) ? key_a : safe_group, kblk, kslots_a[kb]);
             kpage_a[kb] = pl.page(kblk);
-            page_slot(a, key_b >= kv_begin && key_b < kv_end ? key_b : safe_group, kblk, kslots_b[kb]);
+            page_slot(a, span.has(key_b) ? key_b : safe_group, kblk, kslots_b[kb]);
             kpage_b[kb] = pl.page(kblk);
         }
         const bf16* vbase = (const bf16*)a.v_pages + ((size_t)vpage * a.nkv + kvh) * hd * bs + vslot;
@@ -559,7 +623,7 @@ struct WaveAttn {
         }
         // softmax on this lane's 16 scores (keys kt0 + 16g + 4kb + r); the row's four lanes share max and sum
         uint4 p_lo, p_hi;
-        const float alpha = softmax_step<true>(sc, kt0 + 16 * g, lo, hi, a.scale * LOG2E, m, l, p_lo, p_hi);
+        const float alpha = softmax_step<true>(sc, kt0 + 16 * g, lo, hi, a.scale * LOG2E, m, l, p_lo, p_hi, span.keep);
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
         float al[4] = {1.f, 1.f, 1.f, 1.f};
         if (rescale) {
@@ -584,8 +648,8 @@ struct WaveAttn {
                 v1 = and_mask(swap_halves<0x3>(t2, t1), ok);
             }
             if (edge) {
-                v0 = keep_keys(v0, kg, kv_begin, kv_end);
-                v1 = keep_keys(v1, kg + 8, kv_begin, kv_end);
+                v0 = keep_keys(v0, kg, span);
+                v1 = keep_keys(v1, kg + 8, span);
             }
             o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, v0, v1);
         }
@@ -614,16 +678,19 @@ __global__ __launch_bounds__(64) void attn_mfma_tile_kernel(AttnArgs a) {
     WaveAttn<HD> w;
     w.init(qrow, hd);
     const PageLookup pl = {bt, nullptr, 0, 0};
-    for (int kt0 = (kv_begin / 64) * 64; kt0 < kv_end; kt0 += 64) w.tile(a, pl, kvh, kt0, kv_begin, kv_end, lo, hi);
+    const KeySpan span = {kv_begin, kv_end, a.keep_first};
+    const TileWalk walk = tile_walk(span);
+    for (int ti = 0; ti < walk.n; ++ti) w.tile(a, pl, kvh, walk.start(ti), span, lo, hi);
+    const float fin = li < n ? finish_row<true>(a, h, w.m, w.l) : 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
-        const float lr = __shfl(w.l, row, 64);
+        const float fr = __shfl(fin, row, 64);
         if (row < n) {
 #pragma unroll
             for (int cb = 0; cb < WaveAttn<HD>::CB; ++cb) {
                 const int d = 16 * cb + li;
-                if (d < hd) from_float((bf16*)a.out + (size_t)(tok0 + row) * a.ldo + (size_t)h * hd + d, w.o[cb][r] / lr);
+                if (d < hd) store_out<bf16>(a, tok0 + row, h, d, w.o[cb][r] * fr);
             }
         }
     }
@@ -681,9 +748,11 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
     const bool row_ok = li < n;
     w.init(row_ok && !empty ? (const bf16*)a.q + (size_t)tok * a.ldq + (size_t)(h0 + li) * hd : nullptr, hd);
     if (!empty) {
+        // (the kept first keys of the sequence, where they lie before the window, go with the first split)
+        const KeySpan span = {kv_begin, kv_end, split == 0 ? min(a.keep_first, kv_begin) : 0};
+        const TileWalk walk = tile_walk(span);
         const int lo = row_ok ? kv_begin : 1, hi = row_ok ? kv_end - 1 : 0;
-        for (int kt0 = (kv_begin / 64) * 64 + wave * 64; kt0 < kv_end; kt0 += n_waves * 64)
-            w.tile(a, pl, kvh, kt0, kv_begin, kv_end, lo, hi);
+        for (int ti = wave; ti < walk.n; ti += n_waves) w.tile(a, pl, kvh, walk.start(ti), span, lo, hi);
     }
     const int stride = HD + 2;
     float* mine = wave_out + (size_t)wave * n * stride;
@@ -713,7 +782,7 @@ __global__ __launch_bounds__(MAX_THREADS) void attn_mfma_decode_block_kernel(Att
         }
         const int h = h0 + row;
         if (a.splits == 1) {
-            from_float((bf16*)a.out + (size_t)tok * a.ldo + (size_t)h * hd + d, o / l);
+            store_out<bf16>(a, tok, h, d, o * finish_row<true>(a, h, m, l));
         } else {
             a.part_o[(((size_t)item * a.nh + h) * a.splits + split) * hd + d] = o;
             if (d == 0) {
@@ -791,6 +860,8 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
     // Loads are issued without branches: a key outside [kv_begin, kv_end) (its page may have been
     // given back) reads from a group of keys that is inside, and its data is replaced by zeros.
     const int safe_group = (kv_end - 1) & ~15;
+    const KeySpan span = {kv_begin, kv_end, a.keep_first};
+    const TileWalk walk = tile_walk(span);
     __shared__ int page_copy[PAGE_COPY];
     int first_blk, last_blk, unused;
     page_slot(a, kv_begin, first_blk, unused);
@@ -802,7 +873,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int key0 = kt0 + 16 * j;
-            live[j] = key0 < kv_end && key0 + 16 > kv_begin;
+            live[j] = span.touches(key0, 16);
             int blk, slot;
             page_slot(a, live[j] ? key0 : safe_group, blk, slot);
             const size_t page = pl.page(blk);
@@ -815,7 +886,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
             if (c < KCH) {
                 const int r = c / (HD / 8), d = (c % (HD / 8)) * 8;
                 const int key = kt0 + r;
-                const bool ok = key >= kv_begin && key < kv_end && d < hd;
+                const bool ok = span.has(key) && d < hd;
                 const uint4 v = *(const uint4*)((const bf16*)a.k_pages + kbase[r >> 4] + (size_t)(r & 15) * hd + (d < hd ? d : 0));
                 kreg[i] = ok ? v : make_uint4(0, 0, 0, 0);
             }
@@ -827,7 +898,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
                 const int d = c >> 3, k8 = (c & 7) * 8;
                 const bool ok = d < hd && live[k8 >> 4];
                 uint4 v = *(const uint4*)((const bf16*)a.v_pages + vbase[k8 >> 4] + (size_t)(d < hd ? d : 0) * bs + (k8 & 15));
-                if (kt0 < kv_begin || kt0 + 64 > kv_end) v = keep_keys(v, kt0 + k8, kv_begin, kv_end);
+                if (!span.holds_tile(kt0)) v = keep_keys(v, kt0 + k8, span);
                 vreg[i] = ok ? v : make_uint4(0, 0, 0, 0);
             }
         }
@@ -849,18 +920,18 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
         }
     };
 
-    const int kt_first = (kv_begin / 64) * 64;
-    fetch(kreg_a, vreg_a, kt_first);
-    if (kt_first + 64 < kv_end) fetch(kreg_b, vreg_b, kt_first + 64);
+    fetch(kreg_a, vreg_a, walk.start(0));
+    if (1 < walk.n) fetch(kreg_b, vreg_b, walk.start(1));
     int parity = 0;
-    for (int kt0 = kt_first; kt0 < kv_end; kt0 += 64, parity ^= 1) {
+    for (int ti = 0; ti < walk.n; ++ti, parity ^= 1) {
+        const int kt0 = walk.start(ti);
         lds_barrier();            // the previous tile has been read by every wave
         if (parity == 0) stage(kreg_a, vreg_a); else stage(kreg_b, vreg_b);
         lds_barrier();
-        if (kt0 + 128 < kv_end) {  // the registers just emptied take the tile after the next
-            if (parity == 0) fetch(kreg_a, vreg_a, kt0 + 128); else fetch(kreg_b, vreg_b, kt0 + 128);
+        if (ti + 2 < walk.n) {     // the registers just emptied take the tile after the next
+            if (parity == 0) fetch(kreg_a, vreg_a, walk.start(ti + 2)); else fetch(kreg_b, vreg_b, walk.start(ti + 2));
         }
-        if (kt0 > w_hi || kt0 + 64 <= w_lo) continue;      // nothing in this tile for this wave's rows
+        if (kt0 > w_hi || (kt0 + 64 <= w_lo && kt0 >= span.keep)) continue;      // nothing in this tile for this wave's rows
         f32x4_t sc[4];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
@@ -875,7 +946,7 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
         const bool whole = kt0 >= w_lo_max && kt0 + 63 <= w_hi_min && kt0 >= kv_begin;
         uint4 p_lo, p_hi;
         const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi)
-                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi);
+                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi, span.keep);
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
         float al[4] = {1.f, 1.f, 1.f, 1.f};
         if (rescale) {
@@ -888,15 +959,16 @@ __global__ __launch_bounds__(256) void attn_mfma_block_kernel(AttnArgs a) {
             o[cb] = pv_step(o[cb], rescale, al, p_lo, p_hi, *(const uint4*)vr, *(const uint4*)(vr + 8));
         }
     }
+    const float fin = li < n ? finish_row<true>(a, h, m, l) : 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
-        const float lr = __shfl(l, row, 64);
+        const float fr = __shfl(fin, row, 64);
         if (row < n) {
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 const int d = 16 * cb + li;
-                if (d < hd) from_float((bf16*)a.out + (size_t)(tok0 + row) * a.ldo + (size_t)h * hd + d, o[cb][r] / lr);
+                if (d < hd) store_out<bf16>(a, tok0 + row, h, d, o[cb][r] * fr);
             }
         }
     }
@@ -984,6 +1056,8 @@ __global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(Att
     page_slot(a, kv_begin, first_blk, unused);
     page_slot(a, kv_end - 1, last_blk, unused);
     const PageLookup pl = stage_pages(bt, page_copy, first_blk, last_blk);
+    const KeySpan span = {kv_begin, kv_end, a.keep_first};
+    const TileWalk walk = tile_walk(span);
 
     // what this lane fetches in each of its wave-loads, relative to the tile's first key / value row 0
     int k_src[NLOAD], v_src[NLOAD];
@@ -1017,37 +1091,36 @@ __global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(Att
 
     // Every wave of the block goes through the same barriers: the loop runs over rounds of G tiles, of which group
     // grp takes tile grp (a round's last tiles may not exist: that group then only keeps step).
-    const int kt_first = (kv_begin / 64) * 64;
-    if (kt_first + 64 * grp < kv_end) issue(kt_first + 64 * grp, 0);
-    if (NS == 3 && kt_first + 64 < kv_end) issue(kt_first + 64, 1);
+    // (tiles are counted along the block's walk: the kept first keys' tiles, then the window's)
+    if (grp < walk.n) issue(walk.start(grp), 0);
+    if (NS == 3 && 1 < walk.n) issue(walk.start(1), 1);
     int stage = 0;
-    for (int round0 = kt_first; round0 < kv_end; round0 += 64 * G, stage = (stage + 1 == NS ? 0 : stage + 1)) {
-        const int kt0 = round0 + 64 * grp;
+    for (int round = 0; round < walk.n; round += G, stage = (stage + 1 == NS ? 0 : stage + 1)) {
+        const int ti = round + grp;
+        const int kt0 = ti < walk.n ? walk.start(ti) : kv_end;      // (no such tile: past the keys)
         // this wave's part of the tile has landed (with three stages the next tile's loads may still fly)
-        if (NS == 3 && kt0 + 64 < kv_end) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLOAD) : "memory");
+        if (NS == 3 && ti + 1 < walk.n) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NLOAD) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();                           // ... everyone's has, and the stage read last is free
-        if (kt0 + 64 * G * (NS - 1) < kv_end) issue(kt0 + 64 * G * (NS - 1), (stage + NS - 1) % NS);
+        if (ti + G * (NS - 1) < walk.n) issue(walk.start(ti + G * (NS - 1)), (stage + NS - 1) % NS);
         bf16* st = tiles + (grp * NS + stage) * TILE;
         // a tile at the edge: values of keys outside become zeros.  Whether any tile of the round is one is the
         // same for all waves, so all of them meet at the barrier behind the zeros.
         bool any_edge = false;
 #pragma unroll
-        for (int q = 0; q < G; ++q) {
-            const int kq = round0 + 64 * q;
-            any_edge = any_edge || (kq < kv_end && (kq < kv_begin || kq + 64 > kv_end));
-        }
+        for (int q = 0; q < G; ++q)
+            any_edge = any_edge || (round + q < walk.n && !span.holds_tile(walk.start(round + q)));
         if (any_edge) {
-            if (kt0 < kv_end && (kt0 < kv_begin || kt0 + 64 > kv_end)) {
+            if (kt0 < kv_end && !span.holds_tile(kt0)) {
                 for (int idx = tid; idx < HD * 64; idx += W * 64) {
                     const int d = idx >> 6, key = idx & 63;
-                    if (kt0 + key < kv_begin || kt0 + key >= kv_end)
+                    if (!span.has(kt0 + key))
                         st[64 * HD + d * 64 + (((key >> 3) ^ ((d >> 1) & 7)) * 8) + (key & 7)].bits = 0;
                 }
             }
             lds_barrier();      // the zeros are in LDS (a bare s_barrier does not wait for this wave's stores) before any wave reads values
         }
-        if (kt0 >= kv_end || kt0 > w_hi || kt0 + 64 <= w_lo) continue;      // no such tile, or nothing in it for this wave's rows
+        if (kt0 >= kv_end || kt0 > w_hi || (kt0 + 64 <= w_lo && kt0 >= span.keep)) continue;      // no such tile, or nothing in it for this wave's rows
         f32x4_t sc[4];
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb) {
@@ -1061,7 +1134,7 @@ __global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(Att
         const bool whole = kt0 >= w_lo_max && kt0 + 63 <= w_hi_min && kt0 >= kv_begin;
         uint4 p_lo, p_hi;
         const float alpha = whole ? softmax_step<false>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi)
-                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi);
+                                  : softmax_step<true>(sc, kt0 + 16 * g, lo, hi, c2, m, l, p_lo, p_hi, span.keep);
         const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
         float al[4] = {1.f, 1.f, 1.f, 1.f};
         if (rescale) {
@@ -1093,6 +1166,7 @@ __global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(Att
         const float mn = fmaxf(m, m1), mu = (mn == NEG_INF) ? 0.f : mn;
         const float f0 = __builtin_amdgcn_exp2f(m - mu), f1 = __builtin_amdgcn_exp2f(m1 - mu);
         l = l * f0 + l1 * f1;
+        m = mn;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const float a0 = __shfl(f0, 4 * g + r, 64), a1 = __shfl(f1, 4 * g + r, 64);      // of the accumulator's row 4 g + r
@@ -1100,14 +1174,14 @@ __global__ __launch_bounds__(W * G * 64, W / 2) void attn_mfma_direct_kernel(Att
             for (int cb = 0; cb < CB; ++cb) o[cb][r] = o[cb][r] * a0 + hand[(2 + 4 * cb + r) * 64 + lane] * a1;
         }
     }
+    const float fin = li < n ? finish_row<true>(a, h, m, l) : 0.f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * g + r;
-        const float lr = __shfl(l, row, 64);
+        const float fr = __shfl(fin, row, 64);
         if (row < n) {
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb)
-                from_float((bf16*)a.out + (size_t)(tok0 + row) * a.ldo + (size_t)h * HD + 16 * cb + li, o[cb][r] / lr);
+            for (int cb = 0; cb < CB; ++cb) store_out<bf16>(a, tok0 + row, h, 16 * cb + li, o[cb][r] * fr);
         }
     }
 }
@@ -1128,7 +1202,9 @@ static bool mfma_ok(int dtype, int hd, int bs, const void* q, long ldq, const vo
 }
 
 // ---------------------------------------------------------------------------
-static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int bs, int window, float scale, int vd = 0, int mask_chunk = 0) {
+static int check_common(const char* who, int dtype, int nh, int nkv, int hd, int bs, int window, float scale, int vd = 0, int mask_chunk = 0,
+                        int keep_first = 0) {
+    FX_REQUIRE(keep_first >= 0 && !(keep_first > 0 && mask_chunk > 0), "%s: kept first keys (%d) go with a window, not with a chunked mask (%d)", who, keep_first, mask_chunk);
     FX_REQUIRE(vd >= 0 && vd <= HD_MAX, "%s: value head size %d is outside 1..%d", who, vd, HD_MAX);
     FX_REQUIRE(mask_chunk >= 0 && !(mask_chunk > 0 && window > 0), "%s: a window (%d) or a chunked mask (%d), not both", who, window, mask_chunk);
     // (the bfloat16 kernels take a row's maximum over the raw scores and scale it once, which is the maximum of
@@ -1154,9 +1230,9 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
                          const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                          const int* positions, const int* item_seq, const int* item_tok, const int* item_n,
                          int n_items, int nh, int nkv, int hd, int bs, int window, float scale, int tile_q,
-                         int vd, int mask_chunk) {
+                         int vd, int mask_chunk, int keep_first, const float* sinks, const void* gate, long ldg) {
     if (vd <= 0) vd = hd;
-    if (check_common("attn_tiles", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk)) return 1;
+    if (check_common("attn_tiles", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk, keep_first)) return 1;
     FX_REQUIRE(tile_q == 64 || (tile_q == 128 && wide_items_ok(dtype, hd, bs) && mfma_ok(dtype, hd, bs, q, ldq, k_pages, v_pages, vd)),
                "attn_tiles: items of %d queries (64, or 128 where fx_attn_tile_queries says so)", tile_q);
     if (n_items <= 0) return 0;
@@ -1166,6 +1242,7 @@ FX_API int fx_attn_tiles(void* stream, int dtype, const void* q, long ldq, void*
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = item_n;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
     a.vd = vd; a.mask_chunk = mask_chunk;
+    a.keep_first = window > 0 ? keep_first : 0; a.sinks = sinks; a.gate = gate; a.ldg = ldg;
     a.bs_shift = log2_or_minus_one(bs);
     a.n_items = n_items;
     dim3 grid(n_items * 4, nh), grid_blocks(8 * ceil_div((long)n_items * nh, 8));     // a wave per 16 queries / a block per item
@@ -1202,7 +1279,8 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
                               const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                               const int* positions, const int* item_seq, const int* item_tok, int n_items,
                               int nh, int nkv, int hd, int bs, int window, float scale,
-                              float* part_o, float* part_ml, int splits, int chunk, int waves, int vd = 0, int mask_chunk = 0) {
+                              float* part_o, float* part_ml, int splits, int chunk, int waves, int vd = 0, int mask_chunk = 0,
+                              int keep_first = 0, const float* sinks = nullptr, const void* gate = nullptr, long ldg = 0) {
     if (vd <= 0) vd = hd;
     AttnArgs a = {};
     a.q = q; a.ldq = ldq; a.out = out; a.ldo = ldo; a.k_pages = k_pages; a.v_pages = v_pages;
@@ -1210,6 +1288,7 @@ static int attn_decode_launch(void* stream, int dtype, const void* q, long ldq, 
     a.item_seq = item_seq; a.item_tok = item_tok; a.item_n = nullptr;
     a.nh = nh; a.nkv = nkv; a.hd = hd; a.bs = bs; a.window = window; a.scale = scale;
     a.vd = vd; a.mask_chunk = mask_chunk;
+    a.keep_first = window > 0 ? keep_first : 0; a.sinks = sinks; a.gate = gate; a.ldg = ldg;
     a.bs_shift = log2_or_minus_one(bs);
     a.part_o = part_o; a.part_ml = part_ml; a.splits = splits; a.chunk = chunk;
     dim3 grid(n_items, nh, splits), grid2(n_items, nh);
@@ -1263,13 +1342,14 @@ FX_API int fx_attn_decode(void* stream, int dtype, const void* q, long ldq, void
                           const void* k_pages, const void* v_pages, const int* block_table, int max_blocks,
                           const int* positions, const int* item_seq, const int* item_tok, int n_items,
                           int nh, int nkv, int hd, int bs, int window, float scale,
-                          float* part_o, float* part_ml, int splits, int chunk, int waves, int vd, int mask_chunk) {
+                          float* part_o, float* part_ml, int splits, int chunk, int waves, int vd, int mask_chunk,
+                          int keep_first, const float* sinks, const void* gate, long ldg) {
     if (attn_decode_check(dtype, nh, nkv, hd, bs, window, scale, splits, chunk)) return 1;
-    if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk)) return 1;
+    if (check_common("attn_decode", dtype, nh, nkv, hd, bs, window, scale, vd, mask_chunk, keep_first)) return 1;
     if (n_items <= 0) return 0;
     return attn_decode_launch(stream, dtype, q, ldq, out, ldo, k_pages, v_pages, block_table, max_blocks, positions,
                               item_seq, item_tok, n_items, nh, nkv, hd, bs, window, scale, part_o, part_ml, splits,
-                              chunk, waves, vd, mask_chunk);
+                              chunk, waves, vd, mask_chunk, keep_first, sinks, gate, ldg);
 }
 
 // ---------------------------------------------------------------------------

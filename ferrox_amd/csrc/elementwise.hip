@@ -42,7 +42,8 @@ FX_API int fx_embed(void* stream, int w_dtype, const void* table, const int* ids
 // ---------------------------------------------------------------------------
 // RMSNorm: y = x * rsqrt(mean(x^2) + eps) * w, multiply order x*s*w
 // (ferrox-core/src/matmul.rs:62-69).  Input rows are float32 (the residual
-// stream), optionally gathered through `rows`; output is T.
+// stream), optionally gathered through `rows`; output is T.  Without a weight (w null) rows are only
+// brought to unit root mean square.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ h, const int* __restrict__ rows,
@@ -59,7 +60,11 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
             const int c = threadIdx.x + i * 256;
             xv[i] = c < H ? x[c] : 0.f;
         }
-        load_strided_as_float<16, 256>(w, w_dtype, threadIdx.x, H, wv);
+        if (w) load_strided_as_float<16, 256>(w, w_dtype, threadIdx.x, H, wv);
+        else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) wv[i] = 1.f;
+        }
 #pragma unroll
         for (int i = 0; i < 16; ++i) ss += xv[i] * xv[i];
         ss = block_sum<4>(ss, red);
@@ -79,7 +84,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
     ss = block_sum<4>(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)H + eps);
     for (int c = threadIdx.x; c < H; c += 256)
-        from_float(out + (size_t)r * H + c, x[c] * scale * load_as_float(w, w_dtype, c));
+        from_float(out + (size_t)r * H + c, x[c] * scale * (w ? load_as_float(w, w_dtype, c) : 1.f));
 }
 
 // Short rows (the heads of q and k, normed one by one): a wave per row, four rows to a block, the row in registers.
@@ -98,7 +103,11 @@ __global__ __launch_bounds__(256) void rmsnorm_short_kernel(const float* __restr
         const int c = lane + i * 64;
         xv[i] = c < H ? x[c] : 0.f;
     }
-    load_strided_as_float<4, 64>(w, w_dtype, lane, H, wv);
+    if (w) load_strided_as_float<4, 64>(w, w_dtype, lane, H, wv);
+    else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wv[i] = 1.f;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) ss += xv[i] * xv[i];
     ss = wave_sum(ss);

@@ -4,7 +4,8 @@
 //
 // Layers with the same need share a group: one pool of page ids and one block
 // table per request.  A group keeps all keys (window -1), the last `window`, or (window -(C + 1)) the keys of
-// the current chunk of C positions.
+// the current chunk of C positions.  A windowed group may also keep the first positions of every sequence
+// (fxc_keep_first): the pages that hold them are never given back by trim.
 // The reference keeps an identical store per layer and never evicts
 // (ferrox-core/src/cache.rs:331-488); here a windowed group gives a page back as
 // soon as every later query is past it.  Rules: a page is in exactly one place
@@ -59,6 +60,7 @@ struct Seq {
 struct Manager {
     int block_size;
     std::vector<int> windows;               // per group, < 0: all keys
+    std::vector<int> keep_first;            // per group: so many first positions of a sequence stay, whatever the window
     std::vector<Pool> pools;
     int n_slots;
     std::vector<int> free_slots;
@@ -92,6 +94,7 @@ FX_API void* fxc_create(int n_groups, const int* windows, const int* num_pages, 
             return nullptr;
         }
         m->windows.push_back(windows[g]);
+        m->keep_first.push_back(0);
         m->pools.emplace_back(num_pages[g]);
     }
     m->n_slots = n_slots;
@@ -101,6 +104,16 @@ FX_API void* fxc_create(int n_groups, const int* windows, const int* num_pages, 
 }
 
 FX_API void fxc_destroy(void* h) { delete (Manager*)h; }
+
+// group g keeps the first n positions of every sequence beside its window; to be set before any request is admitted
+FX_API int fxc_keep_first(void* h, int g, int n) {
+    Manager* m = (Manager*)h;
+    if (g < 0 || g >= (int)m->windows.size() || n < 0) return fail(m, "keep_first: group %d, %d positions", g, n);
+    if (m->windows[g] < 0 && n > 0) return fail(m, "keep_first: group %d has no window", g);
+    if (!m->seqs.empty()) return fail(m, "keep_first: requests are admitted already");
+    m->keep_first[g] = n;
+    return 0;
+}
 FX_API const char* fxc_last_error(void* h) { return ((Manager*)h)->error.c_str(); }
 
 // a state slot and empty block tables; -1 if no slot is free, -2 if already admitted
@@ -176,7 +189,8 @@ FX_API int fxc_trim(void* h, int64_t req) {
         if (first_needed <= 0) continue;
         std::vector<int>& t = s->tables[g];
         const int upto = std::min<int>(first_needed / m->block_size, (int)t.size());
-        for (int b = 0; b < upto; ++b)
+        const int kept = (m->keep_first[g] + m->block_size - 1) / m->block_size;      // pages that hold kept first positions
+        for (int b = kept; b < upto; ++b)
             if (t[b] >= 0) {
                 m->pools[g].give(t[b]);
                 t[b] = -1;

@@ -21,8 +21,8 @@ enum { GATE_SOFTMAX = 0, GATE_SIGMOID = 1 };
 // ferrox-models/src/decoder.rs:2915), optionally with the shared expert's gate
 // logit in column E.
 //   softmax over all E with max subtraction, then the k largest probabilities,
-//   weights = those probabilities, divided by their sum if `renorm`
-//   (ferrox-moe/src/lib.rs:333-355).  Ties: higher probability first, then the
+//   weights = those probabilities, divided by their sum (+ w_eps) if `renorm`
+//   (ferrox-moe/src/lib.rs:333-355), then times w_scale (a constant of the mixture; 1 for none).  Ties: higher probability first, then the
 //   lower expert index (the rule of ferrox-metal/src/gpu.rs:686-699).
 //   GATE_SIGMOID scores each expert with 1/(1+exp(-logit)) instead
 //   (ferrox-moe/src/lib.rs:100-121).
@@ -68,7 +68,7 @@ __device__ __forceinline__ void wave_argmax(float& best, int& bi) {
 
 // selection for one token by one wave; `score` is E floats of LDS owned by the wave
 // (`es`: distance between the logits of neighbouring experts, 1 for a row of a [T, E] matrix)
-__device__ __forceinline__ void select_token(const float* __restrict__ row, float* score, int t, int E, int k, int renorm,
+__device__ __forceinline__ void select_token(const float* __restrict__ row, float* score, int t, int E, int k, int renorm, float w_eps, float w_scale,
                                              int gating, int* __restrict__ ids, float* __restrict__ weights,
                                              float* __restrict__ gate_out, int* ids_copy, long es = 1,
                                              const float* __restrict__ sel_bias = nullptr) {
@@ -125,7 +125,7 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
         if (lane < k) {
             store_shared(ids + t * k + lane, my_id);      // (at device scope: a block of this launch may sort them)
             if (ids_copy) ids_copy[t * k + lane] = my_id;
-            weights[t * k + lane] = renorm ? my_w / wsum : my_w;
+            weights[t * k + lane] = (renorm ? my_w / (wsum + w_eps) : my_w) * w_scale;
         }
         return;
     }
@@ -179,23 +179,23 @@ __device__ __forceinline__ void select_token(const float* __restrict__ row, floa
         __builtin_amdgcn_wave_barrier();
         __threadfence_block();
     }
-    if (lane < k) weights[t * k + lane] = renorm ? my_w / wsum : my_w;
+    if (lane < k) weights[t * k + lane] = (renorm ? my_w / (wsum + w_eps) : my_w) * w_scale;
 }
 
 __global__ __launch_bounds__(256) void router_select_kernel(const float* __restrict__ logits, long ld, long es, int T,
-                                                            int E, int k, int renorm, int gating, int* __restrict__ ids,
+                                                            int E, int k, int renorm, float w_eps, float w_scale, int gating, int* __restrict__ ids,
                                                             float* __restrict__ weights, float* __restrict__ gate_out,
                                                             const float* __restrict__ sel_bias) {
     extern __shared__ float score_all[];   // 4 x E
     const int wave = threadIdx.x >> 6;
     const int t = blockIdx.x * 4 + wave;
     if (t >= T) return;
-    select_token(logits + (size_t)t * ld, score_all + wave * E, t, E, k, renorm, gating, ids, weights, gate_out, nullptr, es,
+    select_token(logits + (size_t)t * ld, score_all + wave * E, t, E, k, renorm, w_eps, w_scale, gating, ids, weights, gate_out, nullptr, es,
                  sel_bias);
 }
 
 // logits of token t and expert e stand at logits[t * ld + e * es] (either of the two may be 1)
-FX_API int fx_router_select(void* stream, const float* logits, long ld, long es, int T, int E, int k, int renorm,
+FX_API int fx_router_select(void* stream, const float* logits, long ld, long es, int T, int E, int k, int renorm, float w_eps, float w_scale,
                             int gating, int* ids, float* weights, float* gate_out, const float* sel_bias) {
     FX_REQUIRE(T >= 0, "router: bad size T=%d", T);
     FX_REQUIRE(ld >= 1 && es >= 1, "router: bad strides %ld, %ld", ld, es);
@@ -205,7 +205,7 @@ FX_API int fx_router_select(void* stream, const float* logits, long ld, long es,
                ld, E + (gate_out ? 1 : 0));
     FX_REQUIRE(gating == GATE_SOFTMAX || gating == GATE_SIGMOID, "router: unknown gating %d", gating);
     if (T == 0) return 0;
-    router_select_kernel<<<(T + 3) / 4, 256, 4 * E * sizeof(float), (hipStream_t)stream>>>(logits, ld, es, T, E, k, renorm,
+    router_select_kernel<<<(T + 3) / 4, 256, 4 * E * sizeof(float), (hipStream_t)stream>>>(logits, ld, es, T, E, k, renorm, w_eps, w_scale,
                                                                                          gating, ids, weights, gate_out, sel_bias);
     FX_CHECK_LAUNCH("router_select");
     return 0;
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(SORT_WAVES * 64) void moe_place_kernel(const int* _
 
 // few tokens: selection (a wave per token) and the sort in one block of 16 waves
 __global__ __launch_bounds__(1024) void router_select_align_kernel(const float* __restrict__ logits, long ld, int T, int E,
-                                                                  int k, int renorm, int gating, int* __restrict__ ids,
+                                                                  int k, int renorm, float w_eps, float w_scale, int gating, int* __restrict__ ids,
                                                                   float* __restrict__ weights, float* __restrict__ gate_out,
                                                                   int* __restrict__ expert_offsets,
                                                                   int* __restrict__ sorted_token,
@@ -451,7 +451,7 @@ __global__ __launch_bounds__(1024) void router_select_align_kernel(const float* 
     int* cnt = offs + E + 1;                    // groups x E
     const int wave = threadIdx.x >> 6;
     if (wave < T)
-        select_token(logits + (size_t)wave * ld, score + wave * E, wave, E, k, renorm, gating, ids, weights, gate_out, ids_s);
+        select_token(logits + (size_t)wave * ld, score + wave * E, wave, E, k, renorm, w_eps, w_scale, gating, ids, weights, gate_out, ids_s);
     __syncthreads();
     align_block(ids_s, T * k, k, E, 1, offs, cnt, expert_offsets, sorted_token, sorted_pair, inv);
 }
@@ -485,7 +485,7 @@ __device__ __forceinline__ float dot8(uint4 w, const float* x) {
 #define FRONT_MAX_TOKENS 256
 __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
     const float* __restrict__ h, long ldh, const void* __restrict__ gamma, int gamma_dtype, float eps,
-    bf16* __restrict__ x_out, const bf16* __restrict__ W, int H, int T, int E, int has_gate, int k, int renorm,
+    bf16* __restrict__ x_out, const bf16* __restrict__ W, int H, int T, int E, int has_gate, int k, int renorm, float w_eps, float w_scale,
     int gating, float* logits, int* ids, float* __restrict__ weights, float* __restrict__ gate_out,
     unsigned* counters, int* __restrict__ expert_offsets, int* __restrict__ sorted_token, int* __restrict__ sorted_pair,
     int* __restrict__ inv, int n_always, int per_row) {
@@ -590,7 +590,7 @@ __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
         float* mine = (float*)lds;                  // n_rows logits, then E scores
         for (int e = lane; e < n_rows; e += 64) mine[e] = load_shared(logits + (size_t)t * n_rows + e);
         __builtin_amdgcn_wave_barrier();
-        select_token(mine, mine + n_rows, t, E, k, renorm, gating, ids, weights, has_gate ? gate_out : nullptr, nullptr);
+        select_token(mine, mine + n_rows, t, E, k, renorm, w_eps, w_scale, gating, ids, weights, has_gate ? gate_out : nullptr, nullptr);
     }
     // with a place for the sorted layout: the block that selects the last token sorts all pairs by expert
     if (!expert_offsets) return;
@@ -606,7 +606,7 @@ __global__ __launch_bounds__(FRONT_THREADS) void moe_front_kernel(
 // (T k + n_always T ints) and `inv` (T k, or null) the same launch also sorts the pairs by expert, as
 // fx_moe_align does.
 FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamma, int gamma_dtype, float eps,
-                        void* x_out, const void* W, int H, int T, int E, int has_gate, int k, int renorm, int gating,
+                        void* x_out, const void* W, int H, int T, int E, int has_gate, int k, int renorm, float w_eps, float w_scale, int gating,
                         float* logits, int* ids, float* weights, float* gate_out, unsigned* counters,
                         int* expert_offsets, int* sorted_token, int* sorted_pair, int* inv, int n_always) {
     FX_REQUIRE(T >= 0 && H > 0, "moe_front: bad sizes T=%d H=%d", T, H);
@@ -628,7 +628,7 @@ FX_API int fx_moe_front(void* stream, const float* h, long ldh, const void* gamm
     if (T == 0) return 0;
     dim3 grid(ceil_div(E + has_gate, FRONT_ROWS), T);
     moe_front_kernel<<<grid, FRONT_THREADS, shm, (hipStream_t)stream>>>(h, ldh, gamma, gamma_dtype, eps, (bf16*)x_out,
-                                                                        (const bf16*)W, H, T, E, has_gate, k, renorm,
+                                                                        (const bf16*)W, H, T, E, has_gate, k, renorm, w_eps, w_scale,
                                                                         gating, logits, ids, weights, gate_out, counters,
                                                                         expert_offsets, sorted_token, sorted_pair, inv,
                                                                         n_always, per_row);
@@ -663,7 +663,7 @@ FX_API int fx_moe_align(void* stream, const int* ids, int n, int k, int E, int* 
 
 // Both steps in one launch when the batch is small enough for one block; returns 2 (and
 // launches nothing) when it is not, so that the caller runs the two kernels.
-FX_API int fx_router_select_align(void* stream, const float* logits, long ld, int T, int E, int k, int renorm,
+FX_API int fx_router_select_align(void* stream, const float* logits, long ld, int T, int E, int k, int renorm, float w_eps, float w_scale,
                                   int gating, int* ids, float* weights, float* gate_out, int* expert_offsets,
                                   int* sorted_token, int* sorted_pair, int* inv) {
     FX_REQUIRE(T >= 0, "router: bad size T=%d", T);
@@ -676,7 +676,7 @@ FX_API int fx_router_select_align(void* stream, const float* logits, long ld, in
     const size_t shm = (size_t)(16 * E + n + E + 1) * 4 + (size_t)groups * E * 4;
     if (T > 16 || shm > 48 * 1024) return 2;
     if (T == 0) return 0;
-    router_select_align_kernel<<<1, 1024, shm, (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, gating, ids, weights,
+    router_select_align_kernel<<<1, 1024, shm, (hipStream_t)stream>>>(logits, ld, T, E, k, renorm, w_eps, w_scale, gating, ids, weights,
                                                                      gate_out, expert_offsets, sorted_token, sorted_pair, inv);
     FX_CHECK_LAUNCH("router_select_align");
     return 0;

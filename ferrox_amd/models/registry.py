@@ -83,6 +83,9 @@ def _register_builtin():
     from ..config.rafilix import RafilixConfig
     from .rafilix import build_spec as rafilix_spec
     register_architecture(Architecture(RafilixConfig.architecture, RafilixConfig.model_type, RafilixConfig, rafilix_spec))
+    from ..config.kovalorn import KovalornConfig
+    from .kovalorn import build_spec as kovalorn_spec
+    register_architecture(Architecture(KovalornConfig.architecture, KovalornConfig.model_type, KovalornConfig, kovalorn_spec))
 
 
 _register_builtin()

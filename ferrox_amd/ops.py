@@ -92,18 +92,20 @@ _sigs = {
                               c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
     ("attention", "fx_attn_tiles"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                      c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int],
+                                     c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int,
+                                     c_int, c_void_p, c_void_p, c_long],
     ("attention", "fx_attn_tile_queries"): [c_int, c_int, c_int],
     ("attention", "fx_attn_decode"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                       c_int, c_int, c_int, c_int, c_int, c_float,
-                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int],
-    ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int, c_int, c_int,
+                                      c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                      c_int, c_void_p, c_void_p, c_long],
+    ("moe", "fx_router_select"): [c_void_p, c_void_p, c_long, c_long, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                                   c_void_p, c_void_p, c_void_p, c_void_p],
-    ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_int,
+    ("moe", "fx_router_select_align"): [c_void_p, c_void_p, c_long, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
     ("moe", "fx_moe_front"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_float, c_void_p, c_void_p, c_int, c_int,
-                              c_int, c_int, c_int, c_int, c_int] + [c_void_p] * 9 + [c_int],
+                              c_int, c_int, c_int, c_int, c_float, c_float, c_int] + [c_void_p] * 9 + [c_int],
     ("moe", "fx_moe_align"): [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int],
     ("sampling", "fx_sample_greedy"): [c_void_p, c_void_p, c_long, c_int, c_int, c_void_p, c_void_p, c_void_p],
     ("sampling", "fx_sample"): [c_void_p, c_void_p, c_long, c_void_p, c_int, c_int] + [c_void_p] * 10,
@@ -148,17 +150,18 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor | None = Non
 
 def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
             rows: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
-    """Rows of float32 `h` (all, or those in `rows`) normed into `out_dtype`."""
+    """Rows of float32 `h` (all, or those in `rows`) normed into `out_dtype`; `weight` None: brought to unit root
+    mean square, no more."""
     if h.dtype != torch.float32 or not h.is_contiguous():
         raise KernelError("rmsnorm reads a contiguous float32 residual stream")
     H = h.shape[-1]
-    if weight.numel() != H:
+    if weight is not None and weight.numel() != H:
         raise KernelError(f"rmsnorm weight has {weight.numel()} elements for width {H}")
     R = h.shape[0] if rows is None else rows.numel()
     if out is None:
         out = torch.empty((R, H), dtype=out_dtype, device=h.device)
     _call("elementwise", "fx_rmsnorm", _stream(), dtype_code(out_dtype), _p(h), _p(_i32(rows, "rows")), _p(weight),
-          dtype_code(weight.dtype), _p(out), R, H, float(eps))
+          dtype_code(weight.dtype) if weight is not None else FX_F32, _p(out), R, H, float(eps))
     return out
 
 
@@ -478,17 +481,31 @@ def attention_tile_queries(dtype, head_dim: int, block_size: int) -> int:
 
 def attention_tiles(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok, item_n,
                     n_heads, n_kv_heads, head_dim, block_size, window, scale, tile_q: int = 64, mask_chunk: int = 0,
-                    v_dim: int | None = None) -> None:
+                    v_dim: int | None = None, keep_first: int = 0, sinks=None, gate=None) -> None:
     """Blocks of queries: item i is item_n[i] <= tile_q consecutive tokens of sequence item_seq[i] from token
     item_tok[i] on; tile_q is 64 or attention_tile_queries(...).  `mask_chunk` > 0: the chunked mask (a query sees
     the keys of its own chunk of that many positions) instead of a window.  `v_dim`: size of a value head where it
-    is not head_dim; `out` is [T, n_heads * v_dim]."""
+    is not head_dim; `out` is [T, n_heads * v_dim].  `keep_first` (with a window): the first so many keys of a
+    sequence stay visible to every later query.  `sinks` (float32 [n_heads]): a logit per head that joins the
+    softmax's denominator and has no value.  `gate` (shape and type of `out`): the output is multiplied by sigmoid(gate)."""
     _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, int(v_dim or head_dim), block_size)
+    _check_attention_extras(out, n_heads, int(v_dim or head_dim), window, keep_first, sinks, gate)
     _call("attention", "fx_attn_tiles", _stream(), dtype_code(q.dtype), _p(q), q.stride(0), _p(out), out.stride(0),
           _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")),
           _p(_i32(item_n, "item_n")), item_seq.numel(), n_heads, n_kv_heads, head_dim, block_size,
-          int(window or 0), float(scale), int(tile_q), int(v_dim or head_dim), int(mask_chunk or 0))
+          int(window or 0), float(scale), int(tile_q), int(v_dim or head_dim), int(mask_chunk or 0),
+          int(keep_first or 0), _p(sinks), _p(gate), gate.stride(0) if gate is not None else 0)
+
+
+def _check_attention_extras(out, n_heads, v_dim, window, keep_first, sinks, gate) -> None:
+    if keep_first and not window:
+        raise KernelError("attention: kept first keys go with a window")
+    if sinks is not None and (sinks.dtype != torch.float32 or not sinks.is_contiguous() or sinks.numel() != n_heads):
+        raise KernelError(f"attention: sinks must be {n_heads} contiguous float32 values")
+    if gate is not None and (gate.dtype != out.dtype or gate.stride(-1) != 1 or gate.shape[0] < out.shape[0]
+                             or gate.shape[1] < n_heads * v_dim):
+        raise KernelError(f"attention: gate {tuple(gate.shape)} ({gate.dtype}) for an output {tuple(out.shape)} ({out.dtype})")
 
 
 def _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, v_dim, block_size) -> None:
@@ -530,7 +547,8 @@ def decode_attention_chunk(n_items: int, n_heads: int, n_kv_heads: int, max_kv_l
 
 def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq, item_tok,
                      n_heads, n_kv_heads, head_dim, block_size, window, scale, max_kv_len, chunk=None,
-                     waves=0, mask_chunk: int = 0, v_dim: int | None = None) -> None:
+                     waves=0, mask_chunk: int = 0, v_dim: int | None = None, keep_first: int = 0, sinks=None,
+                     gate=None) -> None:
     """Single queries.  The keys go to ceil(max_kv_len / chunk) blocks whose results are merged in ascending
     order.  float32 cuts them at multiples of `chunk`, 256 by default (so that a result does not depend on the
     batch); bfloat16, whose blocks of up to eight waves share a chunk, cuts every sequence's own range of keys (from
@@ -539,6 +557,7 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
     n = item_seq.numel()
     v_dim = int(v_dim or head_dim)
     _check_attention_shapes(q, out, k_pages, v_pages, n_heads, n_kv_heads, head_dim, v_dim, block_size)
+    _check_attention_extras(out, n_heads, v_dim, window, keep_first, sinks, gate)
     if chunk is None:
         chunk = 256
         if q.dtype == torch.bfloat16:
@@ -550,14 +569,17 @@ def attention_decode(q, out, k_pages, v_pages, block_table, positions, item_seq,
           _p(k_pages), _p(v_pages), _p(_i32(block_table, "block_table")), block_table.shape[1],
           _p(_i32(positions, "positions")), _p(_i32(item_seq, "item_seq")), _p(_i32(item_tok, "item_tok")), n,
           n_heads, n_kv_heads, head_dim, block_size, int(window or 0), float(scale),
-          _p(part_o), _p(part_ml), splits, chunk, int(waves), v_dim, int(mask_chunk or 0))
+          _p(part_o), _p(part_ml), splits, chunk, int(waves), v_dim, int(mask_chunk or 0),
+          int(keep_first or 0), _p(sinks), _p(gate), gate.stride(0) if gate is not None else 0)
 
 
-def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False, selection_bias=None):
+def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False, selection_bias=None,
+                  weighting=(0.0, 1.0)):
     """From float32 router logits [T, >= E (+1)] (any strides, so also the transpose of an
     [E (+1), T] product): (ids int32 [T,k], weights float32 [T,k], gate float32 [T] =
     sigmoid(logits[:, E]) or None).  `selection_bias` (float32 [E]): the experts are chosen by score + bias,
-    the weights are the scores."""
+    the weights are the scores.  `weighting` = (eps, scale): a renormalised weight is score / (sum of the chosen
+    scores + eps), and every weight is multiplied by scale."""
     if selection_bias is not None and (selection_bias.dtype != torch.float32 or not selection_bias.is_contiguous()
                                        or selection_bias.numel() != n_experts):
         raise KernelError(f"router_select: the selection bias must be {n_experts} contiguous float32 values")
@@ -570,11 +592,12 @@ def router_select(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gat
     if logits.shape[1] < n_experts + (1 if has_gate else 0):
         raise KernelError(f"router_select: {logits.shape[1]} columns for {n_experts} experts")
     _call("moe", "fx_router_select", _stream(), _p(logits), logits.stride(0), logits.stride(1), T, n_experts, top_k,
-          1 if renorm else 0, gating, _p(ids), _p(weights), _p(gate), _p(selection_bias))
+          1 if renorm else 0, float(weighting[0]), float(weighting[1]), gating, _p(ids), _p(weights), _p(gate),
+          _p(selection_bias))
     return ids, weights, gate
 
 
-def route(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False):
+def route(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False, weighting=(0.0, 1.0)):
     """router_select followed by moe_align; one launch when the batch is small.
     Returns (ids, weights, gate, expert_offsets, sorted_token, sorted_pair, inv)."""
     if logits.dtype != torch.float32 or logits.dim() != 2:
@@ -589,13 +612,14 @@ def route(logits, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False)
         offsets = torch.empty((n_experts + 1,), dtype=torch.int32, device=dev)
         buf = torch.empty((3, n), dtype=torch.int32, device=dev)
         f, handle = _fn("moe", "fx_router_select_align")
-        rc = f(_stream(), _p(logits), logits.stride(0), T, n_experts, top_k, 1 if renorm else 0, gating, _p(ids),
+        rc = f(_stream(), _p(logits), logits.stride(0), T, n_experts, top_k, 1 if renorm else 0, float(weighting[0]),
+               float(weighting[1]), gating, _p(ids),
                _p(weights), _p(gate), _p(offsets), _p(buf[0]), _p(buf[1]), _p(buf[2]))
         if rc == 0:
             return ids, weights, gate, offsets, buf[0], buf[1], buf[2]
         if rc != 2:
             raise KernelError(handle.fx_last_error().decode())
-    ids, weights, gate = router_select(logits, n_experts, top_k, renorm, gating, has_gate)
+    ids, weights, gate = router_select(logits, n_experts, top_k, renorm, gating, has_gate, weighting=weighting)
     return (ids, weights, gate) + moe_align(ids, n_experts)
 
 
@@ -616,7 +640,7 @@ def _counter(device, n: int = 1) -> torch.Tensor:
 
 
 def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE_SOFTMAX, has_gate=False,
-              align: int | None = None):
+              align: int | None = None, weighting=(0.0, 1.0)):
     """For up to 256 rows of the float32 residual stream, in one launch: RMSNorm into bfloat16, router
     products and selection.  Returns None for sizes the kernel does not take, else
     (x, ids, weights, gate, aligned).  `align` = S asks the same launch for what `moe_align(ids, n_experts,
@@ -638,11 +662,12 @@ def moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating=GATE
         buf = torch.empty((3, T * top_k + align * T), dtype=torch.int32, device=dev)
     f, handle = _fn("moe", "fx_moe_front")
     rc = f(_stream(), _p(h), h.stride(0), _p(norm_weight), dtype_code(norm_weight.dtype), float(eps), _p(x), _p(router),
-           H, T, n_experts, 1 if has_gate else 0, top_k, 1 if renorm else 0, gating, _p(logits), _p(ids), _p(weights),
+           H, T, n_experts, 1 if has_gate else 0, top_k, 1 if renorm else 0, float(weighting[0]), float(weighting[1]),
+           gating, _p(logits), _p(ids), _p(weights),
            _p(gate), _p(_counter(dev, T + 1)), _p(offsets), _p(buf[0]) if buf is not None else None,
            _p(buf[1]) if buf is not None else None, _p(buf[2]) if buf is not None else None, int(align or 0))
     if rc == 2 and align is not None:      # the sort's counters do not fit beside the front's: without it
-        return moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating, has_gate)
+        return moe_front(h, norm_weight, eps, router, n_experts, top_k, renorm, gating, has_gate, weighting=weighting)
     if rc == 2:
         return None
     if rc:

@@ -63,19 +63,28 @@ class PagedAttention(Mixer):
     takes_post_norm = True     # forward(..., post_norm=(weight, eps)) norms the output rows before they join the stream
     TENSORS = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
                "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias",
-               "q_norm": "q_norm.", "k_norm": "k_norm."}
+               "q_norm": "q_norm.", "k_norm": "k_norm.", "sink": "sinks", "gate": "gate_proj.weight"}
 
     def __init__(self, hidden_size: int, n_heads: int, n_kv_heads: int, head_dim: int, bias: bool,
                  position: PartSpec, window: int | None = None, scale: float | None = None,
                  qk_norm: PartSpec | None = None, v_dim: int | None = None, chunk: int | None = None,
-                 names: dict | None = None):
+                 names: dict | None = None, keep_first: int = 0, sink: bool = False, out_gate: bool = False,
+                 own_kv: bool = True, retain: tuple | None = None):
         """`qk_norm`: kind and arguments of a norm over head_dim; two of them are built, with tensors under
         `q_norm.` and `k_norm.`, and applied to every head of q and of k before the rotation.
         `v_dim`: size of a value head where it differs from head_dim (the size of a query and key head).
         `chunk`: a query at position p sees the keys t <= p of its own chunk only, floor(t / chunk) == floor(p / chunk),
         chunks counted from position 0 of the sequence.
         `names`: what the checkpoint calls this part's tensors, where that differs from `TENSORS` (the prefixes of
-        the two norms among them)."""
+        the two norms among them).
+        `keep_first` (with a window): the first so many keys of a sequence stay visible to every later query.
+        `sink`: a learned logit per head ([n_heads]) joins the softmax's denominator; it has no key and no value.
+        `out_gate`: the heads' outputs are multiplied by sigmoid(W_g x), x the mixer's input, before the output
+        projection (W_g: [n_heads * v_dim, hidden]).
+        `own_kv` False: the mixer has no key and value projections and writes no cache; its schedule entry reads
+        the cache of an entry that has them (with these head counts and sizes).
+        `retain` = (window or None, keep_first): how the pages of this mixer's cache group age, where that is not
+        its own mask: the longest window and the most kept keys among the mixers that read the same cache."""
         if n_heads % n_kv_heads:
             raise ValueError(f"n_heads {n_heads} is not a multiple of n_kv_heads {n_kv_heads}")
         # (the matrix-unit kernels take multiples of HEAD_DIM_STEP; other sizes run on the kernels for any shape)
@@ -87,6 +96,17 @@ class PagedAttention(Mixer):
         self.chunk = int(chunk) if chunk else None
         if self.window and self.chunk:
             raise ValueError("an attention layer has a sliding window or a chunked mask, not both")
+        self.keep_first = int(keep_first or 0) if self.window else 0
+        if self.keep_first < 0:
+            raise ValueError(f"keep_first {keep_first} is negative")
+        self.has_sink, self.out_gate, self.own_kv = bool(sink), bool(out_gate), bool(own_kv)
+        if self.chunk and (retain is not None or keep_first):
+            raise ValueError("kept first keys and a retention of their own go with a window, not with a chunked mask")
+        # (None, 0): every key is kept; (W, F): the last W and the first F
+        self.retain = (self.window, self.keep_first) if retain is None else (int(retain[0]) if retain[0] else None, int(retain[1] or 0))
+        if self.retain[0] is not None and (self.window is None or self.window > self.retain[0] or self.keep_first > self.retain[1]):
+            raise ValueError(f"a cache that keeps the last {self.retain[0]} and the first {self.retain[1]} keys does not hold "
+                             f"what a window of {self.window} with {self.keep_first} kept keys sees")
         self.v_dim = int(v_dim) if v_dim else head_dim
         if not 1 <= self.v_dim <= limits.HEAD_DIM_MAX:
             raise ValueError(f"v_dim {self.v_dim}: the attention kernels take up to {limits.HEAD_DIM_MAX}")
@@ -95,12 +115,18 @@ class PagedAttention(Mixer):
         if not 0.0 < self.scale < math.inf:
             raise ValueError(f"the scale of the attention scores must be positive and finite, got {self.scale}")
         self.position = POSITION_ENCODINGS.build(position)
+        if not self.own_kv and (bias or (self.position.rotary() or Rotary(1, 1.0)).rotary_dim):
+            raise ValueError("a mixer that reads another mixer's keys and values has neither biases nor a rotation here")
         self._position_prefix = position.prefix or ""       # where the encoding's own tensors (if any) are named
         self.qw, self.kvw, self.vw, self.ow = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * self.v_dim, n_heads * self.v_dim
-        self.qkv = self.o_proj = None
+        if not self.own_kv:
+            self.kvw = self.vw = 0       # (no rows of k and v in the mixer's matrix)
+        self.qkv = self.o_proj = self.sinks = None
         self.q_norm = self.k_norm = None
         if qk_norm is not None:
             self.q_norm, self.k_norm = (NORMS.build(PartSpec(qk_norm.kind, dict(qk_norm.args))) for _ in range(2))
+        if bias and out_gate:
+            raise ValueError("an attention layer with an output gate has no biases here")
 
     def children(self):
         norms = [(self.names["q_norm"], self.q_norm), (self.names["k_norm"], self.k_norm)] if self.q_norm is not None else []
@@ -108,21 +134,32 @@ class PagedAttention(Mixer):
 
     def param_specs(self):
         H, n = self.hidden_size, self.names
-        specs = {n["q"]: ParamSpec((self.qw, H)), n["k"]: ParamSpec((self.kvw, H)),
-                 n["v"]: ParamSpec((self.vw, H)), n["o"]: ParamSpec((H, self.ow))}
+        specs = {n["q"]: ParamSpec((self.qw, H)), n["o"]: ParamSpec((H, self.ow))}
+        if self.own_kv:
+            specs.update({n["k"]: ParamSpec((self.kvw, H)), n["v"]: ParamSpec((self.vw, H))})
         if self.bias:
             specs.update({n["q_bias"]: ParamSpec((self.qw,)), n["k_bias"]: ParamSpec((self.kvw,)),
                           n["v_bias"]: ParamSpec((self.vw,))})
+        if self.has_sink:
+            specs[n["sink"]] = ParamSpec((self.n_heads,))
+        if self.out_gate:
+            specs[n["gate"]] = ParamSpec((self.ow, H))
         return specs
 
     def load(self, fetch):
+        # one matrix: the rows of q, then (a mixer with projections of its own) of k and v, then of the output gate
         n = self.names
-        w = torch.cat(same_dtype([fetch(n["q"]), fetch(n["k"]), fetch(n["v"])]), dim=0)
+        rows = [fetch(n["q"])] + ([fetch(n["k"]), fetch(n["v"])] if self.own_kv else []) \
+            + ([fetch(n["gate"])] if self.out_gate else [])
+        w = torch.cat(same_dtype(rows), dim=0)
         b = None
         if self.bias:
             b = torch.cat(same_dtype([fetch(n["q_bias"]), fetch(n["k_bias"]), fetch(n["v_bias"])]), dim=0)
         self.qkv = Linear(w, b)
         self.o_proj = Linear(fetch(n["o"]))
+        if self.has_sink:
+            self.sinks = fetch(n["sink"]).float().contiguous()
+
 
     def page_shapes(self, block_size: int) -> dict:
         return {"k": (self.n_kv_heads, block_size, self.head_dim),
@@ -131,14 +168,17 @@ class PagedAttention(Mixer):
     def cache_group(self):
         if self.chunk:      # pages age with the chunks: those of a chunk that has ended are given back
             return ("chunk", self.chunk), ("chunk", self.chunk)
-        return super().cache_group()
+        window, keep = self.retain
+        if window and keep:      # the last `window` keys and the first `keep`
+            return ("window", window, "keep", keep), ("keep", window, keep)
+        return (("window", window), window) if window else (("full",), None)
 
     def forward_from_residual(self, norm, ctx, cache, residual) -> bool:
         """Few tokens: the norm is applied inside the q/k/v product (up to 16 rows it saves a launch; with
         more, every block's reading and norming of all rows costs more than the norm kernel)."""
         rms = norm.rms_params()
         if (ctx.act_dtype != torch.bfloat16 or rms is None or residual.shape[0] > 16 or self.q_norm is not None
-                or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
+                or not self.own_kv or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
             return False
         debug.region("qkv")
         qkv = ops.gemm(residual, self.qkv.weight, bias=self.qkv.bias, norm=rms)
@@ -148,8 +188,8 @@ class PagedAttention(Mixer):
     def takes_scale_later(self, act_dtype) -> bool:
         """Whether forward takes an ops.ScaleLater as x (the block before then leaves its rows that way)."""
         w = self.qkv.weight
-        return (self.q_norm is None and act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and w.shape[1] % 8 == 0
-                and w.data_ptr() % 16 == 0)
+        return (self.q_norm is None and self.own_kv and act_dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+                and w.shape[1] % 8 == 0 and w.data_ptr() % 16 == 0)
 
     def tile_queries(self, ctx, dtype, block_size: int) -> int:
         """Queries per work item of this step's prompt portions: 64, or 128 where the kernel takes that many (a block
@@ -179,14 +219,16 @@ class PagedAttention(Mixer):
         return widest if large <= cus or even_blocks >= EVEN_BLOCKS_PER_CU * cus else 64
 
     def normed_heads(self, x, ctx):
-        """q [T, qw], k [T, kvw] with every head normed, and v [T, kvw]: the q and k products in float32 (the
-        norms read float32 rows), each head a row of a [T * (nh + nkv), head_dim] matrix that the norm kernels
-        gather their rows from."""
-        T, nh, nkv, hd = ctx.n_tokens, self.n_heads, self.n_kv_heads, self.head_dim
+        """q [T, qw], k [T, kvw] with every head normed, and the rest of the product, [T, vw (+ ow)]: v and the
+        output gate's rows.  The q and k products are made in float32 (the norms read float32 rows), each head a
+        row of a [T * (nh + nkv), head_dim] matrix that the norm kernels gather their rows from.  A mixer without
+        projections of its own has no k and no v."""
+        T, nh, hd = ctx.n_tokens, self.n_heads, self.head_dim
+        nkv = self.n_kv_heads if self.own_kv else 0
         w, b = self.qkv.weight, self.qkv.bias
         cut = self.qw + self.kvw
         qk = matmul(x, w[:cut], bias=None if b is None else b[:cut], epilogue=ops.EPI_STORE_F32)
-        v = matmul(x, w[cut:], bias=None if b is None else b[cut:])
+        v = matmul(x, w[cut:], bias=None if b is None else b[cut:]) if w.shape[0] > cut else None
 
         def head_rows():
             first = torch.arange(T, dtype=torch.int32, device=qk.device)[:, None] * (nh + nkv)
@@ -197,7 +239,7 @@ class PagedAttention(Mixer):
         q_rows, k_rows = ctx.memo(f"head rows {nh} {nkv}", head_rows)
         heads = qk.view(T * (nh + nkv), hd)
         q = self.q_norm.forward(heads, ctx, rows=q_rows).view(T, self.qw)
-        k = self.k_norm.forward(heads, ctx, rows=k_rows).view(T, self.kvw)
+        k = self.k_norm.forward(heads, ctx, rows=k_rows).view(T, self.kvw) if nkv else None
         return q, k, v
 
     def forward(self, x, ctx, cache, residual, qkv=None, post_norm=None) -> None:
@@ -206,7 +248,7 @@ class PagedAttention(Mixer):
         rot = self.position.rotary()
         debug.region("qkv")
         fused = (qkv is None and self.q_norm is None and rot is not None and rot.frequencies is None
-                 and self.v_dim == self.head_dim
+                 and self.v_dim == self.head_dim and self.own_kv and not self.out_gate
                  and ops.can_qkv_rope(x, self.qkv.weight, ctx.n_tokens, self.head_dim, rot.rotary_dim, rot.interleaved))
         if fused:
             # few tokens: rotation and cache write happen in the product's epilogue
@@ -216,31 +258,41 @@ class PagedAttention(Mixer):
                                rot.freq_factors)
             q = qkv[:, :self.qw]
         else:
+            gate = None
             if self.q_norm is not None:           # every head of q and k through its norm, between bias and rotation
-                q, k, v = self.normed_heads(x, ctx)
+                q, k, rest = self.normed_heads(x, ctx)
                 qkv = q
+                v = rest[:, :self.vw] if rest is not None else None
+                if self.out_gate:
+                    gate = rest[:, self.vw:]
             else:
                 if qkv is None:
                     if isinstance(x, ops.ScaleLater):     # rows of a norm whose scale the product applies
                         qkv = ops.gemm(x.x, self.qkv.weight, bias=self.qkv.bias, row_ss=(x.ss, x.eps))
                     else:
                         qkv = self.qkv(x)
-                q, k, v = qkv[:, :self.qw], qkv[:, self.qw:self.qw + self.kvw], qkv[:, self.qw + self.kvw:]
+                cut = self.qw + self.kvw
+                q, k, v = qkv[:, :self.qw], qkv[:, self.qw:cut], qkv[:, cut:cut + self.vw]
+                if self.out_gate:
+                    gate = qkv[:, cut + self.vw:]
             debug.region("rope + cache write")
-            if rot is None:
-                self.position.apply(q, k, ctx)
-                rot = NO_ROTATION
-            ops.rope_kv_write(q, k, v, ctx.positions, ctx.token_seq, table,
-                              k_pages if cache.writes else None, v_pages if cache.writes else None,
-                              self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot.rotary_dim, rot.theta,
-                              rot.interleaved, rot.freq_factors, frequencies=rot.frequencies, v_dim=self.v_dim)
+            if self.own_kv:       # (a mixer without keys of its own has no rotation either: nothing to do for its q)
+                if rot is None:
+                    self.position.apply(q, k, ctx)
+                    rot = NO_ROTATION
+                ops.rope_kv_write(q, k, v, ctx.positions, ctx.token_seq, table,
+                                  k_pages if cache.writes else None, v_pages if cache.writes else None,
+                                  self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, rot.rotary_dim, rot.theta,
+                                  rot.interleaved, rot.freq_factors, frequencies=rot.frequencies, v_dim=self.v_dim)
         debug.region("attention")
         out = torch.empty((ctx.n_tokens, self.ow), dtype=qkv.dtype, device=qkv.device)
         tile_q = ctx.memo(f"attention tile {self.n_heads} {self.head_dim} {self.v_dim} {cache.block_size} {q.dtype}",
                           lambda: self.tile_queries(ctx, q.dtype, cache.block_size))
         items = ctx.memo(f"attention_items {tile_q}", lambda: attention_items(ctx, tile_q))
         common = (self.n_heads, self.n_kv_heads, self.head_dim, cache.block_size, self.window, self.scale)
-        mask = dict(mask_chunk=self.chunk or 0, v_dim=self.v_dim)
+        # (the gate multiplies the heads' outputs as the attention kernels write them)
+        mask = dict(mask_chunk=self.chunk or 0, v_dim=self.v_dim, keep_first=self.keep_first, sinks=self.sinks,
+                    gate=None if fused else gate)
         if items["n_tiles"]:
             ops.attention_tiles(q, out, k_pages, v_pages, table, ctx.positions,
                                 items["tile_seq"], items["tile_tok"], items["tile_n"], *common, tile_q=tile_q, **mask)

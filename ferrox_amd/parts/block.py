@@ -9,15 +9,19 @@ from .base import BLOCKS, FEED_FORWARDS, MIXERS, NORMS, Block
 
 @BLOCKS.register("prenorm")
 class PreNormBlock(Block):
-    """h += mixer(norm1(h)); h += ffn(norm2(h))   (ferrox-models/src/decoder.rs:1-5, 2155-2173)."""
+    """h += mixer(norm1(h)); h += ffn(norm2(h))   (ferrox-models/src/decoder.rs:1-5, 2155-2173).
+    A layer without a feed-forward has the first half only."""
     slots = {"norm1": NORMS, "mixer": MIXERS, "norm2": NORMS, "ffn": FEED_FORWARDS}
+    optional_slots = ("norm2", "ffn")
 
     def __init__(self, parts: dict, prefixes: dict):
-        self.norm1, self.mixer, self.norm2, self.ffn = parts["norm1"], parts["mixer"], parts["norm2"], parts["ffn"]
+        self.norm1, self.mixer, self.norm2, self.ffn = parts["norm1"], parts["mixer"], parts.get("norm2"), parts.get("ffn")
+        if (self.ffn is None) != (self.norm2 is None):
+            raise ValueError("a pre-norm block has a feed-forward and its norm, or neither")
         self._prefixes = prefixes
 
     def children(self):
-        return [(self._prefixes[s], getattr(self, s)) for s in ("norm1", "mixer", "norm2", "ffn")]
+        return [(self._prefixes[s], getattr(self, s)) for s in ("norm1", "mixer", "norm2", "ffn") if getattr(self, s) is not None]
 
     chains_norms = True     # forward takes `normed` and `then` and returns what the next block may take as `normed`
 
@@ -41,6 +45,8 @@ class PreNormBlock(Block):
             debug.region("norm")
             self.mixer.forward(self.norm1.forward(h, ctx), ctx, cache, h)
         ctx.carry = None
+        if self.ffn is None:
+            return None
         more = {"then_norm": then} if then is not None and self.ffn.norms_after else {}
         if not self.ffn.forward_from_residual(self.norm2, ctx, h, **more):
             debug.region("norm")

@@ -13,22 +13,25 @@ from .linear import Linear, same_dtype
 @FEED_FORWARDS.register("gated_mlp")
 class GatedMLP(FeedForward):
     kernel_libraries = ("gemm",)
+    TENSORS = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
-    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", names: dict | None = None):
+        """`names`: what the checkpoint calls the three matrices, where that differs from `TENSORS`."""
         if activation not in ops.ACTIVATIONS:
             raise ValueError(f"activation '{activation}' is not one of {sorted(ops.ACTIVATIONS)}")
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.activation = activation
+        self.names = dict(self.TENSORS, **(names or {}))
         self.gate_up = self.down = None
 
     def param_specs(self):
-        H, I = self.hidden_size, self.intermediate_size
-        return {"gate_proj.weight": ParamSpec((I, H)), "up_proj.weight": ParamSpec((I, H)),
-                "down_proj.weight": ParamSpec((H, I))}
+        H, I, n = self.hidden_size, self.intermediate_size, self.names
+        return {n["gate"]: ParamSpec((I, H)), n["up"]: ParamSpec((I, H)), n["down"]: ParamSpec((H, I))}
 
     def load(self, fetch):
-        self.gate_up = Linear(torch.cat(same_dtype([fetch("gate_proj.weight"), fetch("up_proj.weight")]), dim=0))
-        self.down = Linear(fetch("down_proj.weight"))
+        n = self.names
+        self.gate_up = Linear(torch.cat(same_dtype([fetch(n["gate"]), fetch(n["up"])]), dim=0))
+        self.down = Linear(fetch(n["down"]))
 
     def output(self, x):
         """The feed-forward's output as float32 [T, H], added to nothing."""

@@ -37,10 +37,18 @@ def side_stream(device) -> torch.cuda.Stream:
 class SparseMoE(FeedForward):
     kernel_libraries = ("elementwise", "gemm", "moe")
     norms_after = True   # forward(..., then_norm=norm) may leave norm(residual) in ctx.carry for the next layer
+    TENSORS = {"router": "gate.weight", "gate": "experts.{}.gate_proj.weight", "up": "experts.{}.up_proj.weight",
+               "down": "experts.{}.down_proj.weight", "shared": "shared_expert.", "shared_gate": "shared_expert_gate.weight",
+               "shared_names": None}
 
     def __init__(self, hidden_size: int, n_experts: int, top_k: int, expert_intermediate_size: int,
                  norm_topk_prob: bool, gating: str = "softmax", shared_intermediate_size: int = 0,
-                 shared_gate: bool = True, activation: str = "silu"):
+                 shared_gate: bool = True, activation: str = "silu", weight_scale: float = 1.0, renorm_eps: float = 0.0,
+                 names: dict | None = None):
+        """`weight_scale`: a constant that every mixture weight is multiplied by.  `renorm_eps`: added to the sum of the
+        chosen scores before the weights are divided by it (with `norm_topk_prob`).  `names`: what the checkpoint calls
+        this part's tensors, where that differs from `TENSORS` ('{}' stands for an expert's number; `shared` is the
+        shared expert's prefix and `shared_names` its own three names)."""
         if not 1 <= top_k <= n_experts:
             raise ValueError(f"top_k {top_k} must lie in 1..{n_experts}")
         if n_experts > limits.MOE_MAX_EXPERTS or top_k > limits.MOE_MAX_TOP_K:
@@ -54,38 +62,41 @@ class SparseMoE(FeedForward):
         self.hidden_size, self.n_experts, self.top_k = int(hidden_size), int(n_experts), int(top_k)
         self.expert_intermediate_size = int(expert_intermediate_size)
         self.norm_topk_prob, self.gating = bool(norm_topk_prob), GATINGS[gating]
-        self.shared = GatedMLP(hidden_size, shared_intermediate_size, activation) if shared_intermediate_size > 0 else None
+        self.weighting = (float(renorm_eps), float(weight_scale))
+        self.names = dict(self.TENSORS, **(names or {}))
+        self.shared = GatedMLP(hidden_size, shared_intermediate_size, activation, names=self.names["shared_names"]) \
+            if shared_intermediate_size > 0 else None
         self.has_shared_gate = bool(shared_gate) and self.shared is not None
         self.router = self.w_gate_up = self.w_down = None
 
     def children(self):
-        return [("shared_expert.", self.shared)] if self.shared is not None else []
+        return [(self.names["shared"], self.shared)] if self.shared is not None else []
 
     def param_specs(self):
-        H, I = self.hidden_size, self.expert_intermediate_size
-        specs = {"gate.weight": ParamSpec((self.n_experts, H))}
+        H, I, n = self.hidden_size, self.expert_intermediate_size, self.names
+        specs = {n["router"]: ParamSpec((self.n_experts, H))}
         for e in range(self.n_experts):
-            specs[f"experts.{e}.gate_proj.weight"] = ParamSpec((I, H))
-            specs[f"experts.{e}.up_proj.weight"] = ParamSpec((I, H))
-            specs[f"experts.{e}.down_proj.weight"] = ParamSpec((H, I))
+            specs[n["gate"].format(e)] = ParamSpec((I, H))
+            specs[n["up"].format(e)] = ParamSpec((I, H))
+            specs[n["down"].format(e)] = ParamSpec((H, I))
         if self.has_shared_gate:
-            specs["shared_expert_gate.weight"] = ParamSpec((1, H))
+            specs[n["shared_gate"]] = ParamSpec((1, H))
         return specs
 
     def load(self, fetch):
-        router = fetch("gate.weight")
+        n = self.names
+        router = fetch(n["router"])
         gu, dn = [], []
         for e in range(self.n_experts):
-            gu.append(torch.cat(same_dtype([fetch(f"experts.{e}.gate_proj.weight"),
-                                            fetch(f"experts.{e}.up_proj.weight")]), dim=0))
-            dn.append(fetch(f"experts.{e}.down_proj.weight"))
+            gu.append(torch.cat(same_dtype([fetch(n["gate"].format(e)), fetch(n["up"].format(e))]), dim=0))
+            dn.append(fetch(n["down"].format(e)))
         # A shared expert whose width is a multiple of the experts' is also kept cut into pieces of their
         # shape, after the experts in the same tensors: for few tokens it then runs as experts that every
         # token takes, inside the experts' two launches (its own copy serves many tokens).
         I, E, H = self.expert_intermediate_size, self.n_experts, self.hidden_size
         self.shared_pieces = 0
         if self.shared is not None and self.shared.intermediate_size % I == 0:
-            sg, su, sdn = (fetch("shared_expert." + n) for n in ("gate_proj.weight", "up_proj.weight", "down_proj.weight"))
+            sg, su, sdn = (fetch(n["shared"] + self.shared.names[m]) for m in ("gate", "up", "down"))
             if all(t.dtype == gu[0].dtype for t in gu + dn + [sg, su, sdn]):
                 S = self.shared.intermediate_size // I
                 for s in range(S):
@@ -103,7 +114,7 @@ class SparseMoE(FeedForward):
         self.w_gate_up_all, self.w_down_all = all_gu, all_dn
         self.w_gate_up, self.w_down = all_gu[:E], all_dn[:E]
         if self.has_shared_gate:     # the gate's row rides along as column E of the router product
-            router = torch.cat(same_dtype([router, fetch("shared_expert_gate.weight").reshape(1, -1)]), dim=0)
+            router = torch.cat(same_dtype([router, fetch(n["shared_gate"]).reshape(1, -1)]), dim=0)
         self.router = router.contiguous()
 
     @staticmethod
@@ -136,7 +147,8 @@ class SparseMoE(FeedForward):
         # pairs, and the launch that selects the experts also sorts the pairs by expert
         S = self.shared_pieces if ctx.act_dtype == self.w_gate_up_all.dtype and T * self.top_k <= 2048 else 0
         front = ops.moe_front(residual, rms[0], rms[1], self.router, self.n_experts, self.top_k,
-                              self.norm_topk_prob, self.gating, self.has_shared_gate, align=None if unsorted else S)
+                              self.norm_topk_prob, self.gating, self.has_shared_gate, align=None if unsorted else S,
+                              weighting=self.weighting)
         if front is None:
             return False
         x, ids, weights, gate, sort = front
@@ -195,7 +207,7 @@ class SparseMoE(FeedForward):
             else:
                 logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
             ids, weights, gate = ops.router_select(logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating,
-                                                   self.has_shared_gate)
+                                                   self.has_shared_gate, weighting=self.weighting)
             S = self.shared_pieces
             self.forward(x, ctx, residual, routed=(ids, weights, gate) + ops.moe_align(ids, self.n_experts, always=S),
                          then_norm=then_norm, sorted_pieces=S)
@@ -222,7 +234,7 @@ class SparseMoE(FeedForward):
             else:
                 logits = matmul(x, self.router, epilogue=ops.EPI_STORE_F32)
             routed = ops.route(logits, self.n_experts, self.top_k, self.norm_topk_prob, self.gating,
-                               self.has_shared_gate)
+                               self.has_shared_gate, weighting=self.weighting)
         ids, weights, gate, offsets, sorted_token, sorted_pair, _ = routed
         if debug.routing_trace is not None:
             debug.routing_trace.put(ids)

@@ -1,5 +1,6 @@
 """RMSNorm (ferrox-core/src/matmul.rs:62-69): y = x * rsqrt(mean(x^2) + eps) * w,
-statistics in float32, read from the float32 residual stream."""
+statistics in float32, read from the float32 residual stream.  A design may store
+its weight around zero (y = ... * (offset + w)), or have none at all."""
 from __future__ import annotations
 
 from .. import ops
@@ -10,21 +11,39 @@ from .base import NORMS, Norm, ParamSpec
 class RMSNorm(Norm):
     kernel_libraries = ("elementwise",)
 
-    def __init__(self, size: int, eps: float, name: str = "weight"):
-        """`name`: what the weight is called behind the part's prefix."""
+    def __init__(self, size: int, eps: float, name: str = "weight", offset: float = 0.0, weight: bool = True,
+                 gain: float = 1.0):
+        """`name`: what the weight is called behind the part's prefix.  `offset`: the stored tensor is the weight
+        minus this number (a weight stored around zero has offset 1); the sum is made once, in float32, and kept in
+        float32, so that nothing of the stored tensor's precision is lost.  `weight` False: no tensor, rows are
+        brought to unit root mean square and no more.  `gain`: a constant that the normed rows are multiplied by (a
+        model that scales its logits by a constant scales the rows in front of its head: the head is linear); it is
+        folded into the float32 weight."""
         self.size = int(size)
         self.eps = float(eps)
         self.name = name
+        self.offset, self.gain = float(offset), float(gain)
+        if not weight and gain != 1.0:
+            raise ValueError("a norm without a weight has no gain")
+        self.has_weight = bool(weight)
         self.weight = None
 
     def param_specs(self):
-        return {self.name: ParamSpec((self.size,), init="ones")}
+        if not self.has_weight:
+            return {}
+        return {self.name: ParamSpec((self.size,), init="zeros" if self.offset else "ones")}
 
     def load(self, fetch):
-        self.weight = fetch(self.name).contiguous()
+        if self.has_weight:
+            w = fetch(self.name)
+            if self.offset or self.gain != 1.0:
+                self.weight = ((w.float() + self.offset) * self.gain).contiguous()
+            else:
+                self.weight = w.contiguous()
 
     def rms_params(self):
-        return self.weight, self.eps
+        """(weight, eps) of a norm that other parts' kernels may apply themselves; a norm without a weight declines."""
+        return (self.weight, self.eps) if self.has_weight else None
 
     def forward(self, h, ctx, rows=None):
         return ops.rmsnorm(h, self.weight, self.eps, ctx.act_dtype, rows=rows)
