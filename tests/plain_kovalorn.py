@@ -60,7 +60,8 @@ def attention(h, w, pre, m, eps, kv):
     H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q = unit_rms((h @ w[pre + "q"].to(F64).T).view(n, H, D), eps)
     k, v = kv
-    see = visible(n, m["mask"]["size"], m["mask"]["keep_first"])
+    mask = m.get("mask")
+    see = visible(n, mask["size"], mask.get("keep_first", 0)) if mask else visible(n, n, 0)
     sink = w[pre + "sink"].to(F64)
     out = torch.zeros(n, H, V, dtype=F64)
     for a in range(H):
@@ -85,12 +86,16 @@ def router_choice(h, w_router, top: int, scale: float):
     return ids, val / (val.sum(-1, keepdim=True) + 1e-20) * scale
 
 
-def mixture(h, w, pre, f, routing=None):
+def mixture(h, w, pre, f, routing=None, margins=None):
     r = f["router"]
     ids, wts = router_choice(h, w[pre + "router"], r["top"], r["scale"])
     if routing is not None:      # the choices of another run; the weights follow from this run's scores
-        ids = routing
-        s = torch.sigmoid(h @ w[pre + "router"].to(F64).T).gather(1, ids.long())
+        all_s = torch.sigmoid(h @ w[pre + "router"].to(F64).T)
+        ids = torch.as_tensor(routing, dtype=torch.long)
+        s = all_s.gather(1, ids)
+        if margins is not None:  # how far below this run's last choice the other run's worst choice scores
+            kth = torch.topk(all_s, r["top"], dim=-1).values[:, -1]
+            margins.append(float((kth - s.min(-1).values).max()))
         wts = s / (s.sum(-1, keepdim=True) + 1e-20) * r["scale"]
     y = torch.zeros_like(h)
     for e in range(r["experts"]):
@@ -102,10 +107,10 @@ def mixture(h, w, pre, f, routing=None):
     return y, ids
 
 
-def forward(cfg: dict, w: dict, tokens, routing=None, layers_out=None):
+def forward(cfg: dict, w: dict, tokens, routing=None, layers_out=None, margins=None):
     """float64 logits [n, vocab] of one sequence.  `routing`: per layer with a mixture, the expert ids to use
-    (from a run whose close calls went the other way).  `layers_out`: a list that receives the stream after
-    every layer."""
+    (from a run whose close calls went the other way); `margins` then receives, per mixture, how far such a choice
+    scores below this run's own.  `layers_out`: a list that receives the stream after every layer."""
     eps = cfg["norm"]["eps"]
     x = w["embed"].to(F64)[torch.as_tensor(tokens, dtype=torch.long)]
     held = {}
@@ -127,12 +132,10 @@ def forward(cfg: dict, w: dict, tokens, routing=None, layers_out=None):
             if f["kind"] == "dense":
                 x = x + gated(h, w, pre + "mlp.", gelu_tanh)
             else:
-                y, ids = mixture(h, w, pre + "mlp.", f, None if routing is None else routing[len(chosen)])
+                y, ids = mixture(h, w, pre + "mlp.", f, None if routing is None else routing[len(chosen)], margins)
                 chosen.append(ids)
                 x = x + y
         if layers_out is not None:
             layers_out.append(x.clone())
     x = offset_norm(x, w["final.norm"].to(F64), eps)
-    logits = (x @ w["embed"].to(F64).T) * cfg["logit_scale"]
-    forward.last_routing = chosen
-    return logits
+    return (x @ w["embed"].to(F64).T) * cfg.get("logit_scale", 1.0)
