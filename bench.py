@@ -405,7 +405,7 @@ def run_workload(name: str, args) -> int:
     return 0
 
 
-# ---- Rafilix beside the closest existing model, at equal layer sizes ------------------------------------------------
+# ---- Rafilix and Kovalorn beside the closest existing model, at equal layer sizes ----------------------------------
 # Layer sizes that resemble a real model's; every model is four layers of random weights.  The Rafilix layers are
 # measured by kind (all attention, all recurrent) and in the design's usual mixture, the Qwen2-MoE layers have the
 # same width, heads, experts and expert width and no shared expert (Rafilix has none).
@@ -432,8 +432,25 @@ def design_configs(s: dict) -> dict:
                 head_dim=s["dim"], num_experts=s["experts"], num_experts_per_tok=s["top"], moe_intermediate_size=s["ff"],
                 shared_expert_intermediate_size=0, vocab_size=s["vocab"], num_hidden_layers=4, max_position_embeddings=16384,
                 tie_word_embeddings=True)
+    # Kovalorn: gated attention under a window beside kept first keys, sigmoid-scored experts with a shared expert
+    # of twice an expert's width; beside it Qwen2-MoE layers with a shared expert of that width.  In the second
+    # variant the last two layers read the second layer's keys and values.
+    def kovalorn(readers):
+        kmlp = {"kind": "moe", "expert": {"ff": s["ff"]}, "router": {"experts": s["experts"], "top": s["top"], "scale": 2.5},
+                "shared": {"ff": 2 * s["ff"]}}
+        layers = []
+        for i in range(4):
+            mixer = {"heads": s["heads"], "kv_heads": s["kv_heads"], "dim": s["dim"], "vdim": s["dim"], "scale": s["dim"] ** -0.5,
+                     "mask": {"size": 8192, "keep_first": 64}}
+            if i in readers:
+                mixer["kv_from"] = 1
+            layers.append({"type": "attention", "mixer": mixer, "mlp": kmlp})
+        return {"architecture": "Kovalorn", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-5}, "logit_scale": 1.0,
+                "layers": layers, "max_positions": 16384}
     return {"qwen2-moe": qwen, "rafilix attention": rafilix([attn] * 4), "rafilix recurrent": rafilix([delta] * 4),
-            "rafilix mixed": rafilix([attn, delta, delta, attn])}
+            "rafilix mixed": rafilix([attn, delta, delta, attn]),
+            "qwen2-moe shared expert": dict(qwen, shared_expert_intermediate_size=2 * s["ff"]),
+            "kovalorn": kovalorn(()), "kovalorn shared keys": kovalorn((2, 3))}
 
 
 def compare_designs(args) -> int:
@@ -725,7 +742,8 @@ def main() -> int:
                     help="per-kernel times of one workload, measured by rocprofv3 around a child process")
     ap.add_argument("--out", help="with --kernel-table: also write the table to this file")
     ap.add_argument("--compare-designs", action="store_true",
-                    help="Rafilix layers (all attention, all recurrent, mixed) beside Qwen2-MoE layers of equal sizes: "
+                    help="Rafilix layers (all attention, all recurrent, mixed) and Kovalorn layers (with keys of their own, "
+                         "reading another layer's) beside Qwen2-MoE layers of equal sizes: "
                          "prefill of --ctx tokens, decode at batch 1 and --batch; random weights, four layers each")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), help="with --compare-designs: one size only")
     ap.add_argument("--design", help="with --compare-designs: only the designs whose name holds this text")

@@ -155,6 +155,42 @@ FX_API int fx_rmsnorm(void* stream, int out_dtype, const float* h, const int* ro
 // [page][kv_head][value head size][slot], which is what the attention kernels read (a value head's size vd
 // may differ from head_dim, the size of a query and key head).
 // ---------------------------------------------------------------------------
+// Values into their transposed pages: block b of ceil(T / 8) * nkv takes eight consecutive tokens of one kv head, so
+// that eight tokens that follow each other in one page go out as one 16-byte store per head dimension.
+template <typename T>
+__device__ __forceinline__ void write_values(int b, const T* __restrict__ v, int ldv, const int* __restrict__ positions,
+                                             const int* __restrict__ token_seq, const int* __restrict__ block_table,
+                                             int max_blocks, T* __restrict__ v_pages, int n_tokens, int nkv, int bs, int vd) {
+    const int tid = threadIdx.x;
+    const int kh = b % nkv, t0 = (b / nkv) * 8;
+    const int n = min(8, n_tokens - t0);
+    const int pos0 = positions[t0], seq0 = token_seq[t0];
+    bool together = sizeof(T) == 2 && n == 8 && (bs & 7) == 0 && (pos0 & 7) == 0;
+    for (int i = 1; together && i < 8; ++i) together = positions[t0 + i] == pos0 + i && token_seq[t0 + i] == seq0;
+    if (together) {
+        const int page = block_table[(size_t)seq0 * max_blocks + pos0 / bs];
+        T* dst = v_pages + ((size_t)page * nkv + kh) * vd * bs + pos0 % bs;
+        for (int d = tid; d < vd; d += 256) {
+            uint16_t e[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) e[i] = *(const uint16_t*)(v + (size_t)(t0 + i) * ldv + (size_t)kh * vd + d);
+            uint4 o;
+            o.x = e[0] | ((uint32_t)e[1] << 16);
+            o.y = e[2] | ((uint32_t)e[3] << 16);
+            o.z = e[4] | ((uint32_t)e[5] << 16);
+            o.w = e[6] | ((uint32_t)e[7] << 16);
+            *(uint4*)(dst + (size_t)d * bs) = o;
+        }
+        return;
+    }
+    for (int idx = tid; idx < n * vd; idx += 256) {      // tokens of different pages: element by element
+        const int i = idx / vd, d = idx - i * vd;
+        const int t = t0 + i, pos = positions[t];
+        const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
+        v_pages[(((size_t)page * nkv + kh) * vd + d) * bs + pos % bs] = v[(size_t)t * ldv + (size_t)kh * vd + d];
+    }
+}
+
 // The first T * split blocks rotate: `split` blocks share a token, each computes the angles' sines
 // and cosines once and takes its part of the heads of q (in place) and of k (into its page); few
 // tokens get several blocks each, many tokens one.  The blocks after them write v: one block per (eight
@@ -235,34 +271,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         return;
     }
     if (!v_pages) return;
-    const int b = blockIdx.x - n_tokens * split;
-    const int kh = b % nkv, t0 = (b / nkv) * 8;
-    const int n = min(8, n_tokens - t0);
-    const int pos0 = positions[t0], seq0 = token_seq[t0];
-    bool together = sizeof(T) == 2 && n == 8 && (bs & 7) == 0 && (pos0 & 7) == 0;
-    for (int i = 1; together && i < 8; ++i) together = positions[t0 + i] == pos0 + i && token_seq[t0 + i] == seq0;
-    if (together) {
-        const int page = block_table[(size_t)seq0 * max_blocks + pos0 / bs];
-        T* dst = v_pages + ((size_t)page * nkv + kh) * vd * bs + pos0 % bs;
-        for (int d = tid; d < vd; d += 256) {
-            uint16_t e[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) e[i] = *(const uint16_t*)(v + (size_t)(t0 + i) * ldv + (size_t)kh * vd + d);
-            uint4 o;
-            o.x = e[0] | ((uint32_t)e[1] << 16);
-            o.y = e[2] | ((uint32_t)e[3] << 16);
-            o.z = e[4] | ((uint32_t)e[5] << 16);
-            o.w = e[6] | ((uint32_t)e[7] << 16);
-            *(uint4*)(dst + (size_t)d * bs) = o;
-        }
-        return;
-    }
-    for (int idx = tid; idx < n * vd; idx += 256) {      // tokens of different pages: element by element
-        const int i = idx / vd, d = idx - i * vd;
-        const int t = t0 + i, pos = positions[t];
-        const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
-        v_pages[(((size_t)page * nkv + kh) * vd + d) * bs + pos % bs] = v[(size_t)t * ldv + (size_t)kh * vd + d];
-    }
+    write_values<T>(blockIdx.x - n_tokens * split, v, ldv, positions, token_seq, block_table, max_blocks, v_pages, n_tokens, nkv, bs, vd);
 }
 
 FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const void* k, int ldk,
@@ -297,6 +306,87 @@ FX_API int fx_rope_kv_write(void* stream, int dtype, void* q, int ldq, const voi
     else
         return fx_fail("rope_kv_write: unknown dtype %d", dtype);
     FX_CHECK_LAUNCH("rope_kv_write");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// Mixers whose q and k heads go through an RMS norm and are not rotated: one launch norms every head of the
+// float32 q/k product, writes q in the activation type, k into its page and v into its transposed page.
+//   qk [T, (nh + nkv) * hd] float32: per token nh heads of q, then nkv heads of k (nkv_in = 0: no keys, q alone).
+//   y = x / sqrt(mean(x^2) + eps) (* w[d] with a weight of hd elements; wq for q's heads, wk for k's).
+// A wave per (token, head), four to a block, the head in registers (hd <= 256): the same sums in the same order as
+// the norm kernel for short rows.  The blocks after them write v (write_values).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_kv_write_kernel(
+    const float* __restrict__ qk, long ldqk, T* __restrict__ q_out, long ldq, const T* __restrict__ v, int ldv,
+    const void* __restrict__ wq, const void* __restrict__ wk, int w_dtype, float eps,
+    const int* __restrict__ positions, const int* __restrict__ token_seq, const int* __restrict__ block_table, int max_blocks,
+    T* __restrict__ k_pages, T* __restrict__ v_pages, int n_tokens, int nh, int nkv, int hd, int bs, int vd, int norm_blocks) {
+    if ((int)blockIdx.x >= norm_blocks) {
+        if (v_pages) write_values<T>(blockIdx.x - norm_blocks, v, ldv, positions, token_seq, block_table, max_blocks, v_pages, n_tokens, nkv, bs, vd);
+        return;
+    }
+    const int heads = nh + (k_pages ? nkv : 0);
+    const int r = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (r >= n_tokens * heads) return;
+    const int t = r / heads, head = r - t * heads;
+    const float* x = qk + (size_t)t * ldqk + (size_t)head * hd;
+    const void* w = head < nh ? wq : wk;
+    float xv[4], wv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = lane + i * 64;
+        xv[i] = c < hd ? x[c] : 0.f;
+    }
+    if (w) load_strided_as_float<4, 64>(w, w_dtype, lane, hd, wv);
+    else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) wv[i] = 1.f;
+    }
+    T* dst;
+    if (head < nh) dst = q_out + (size_t)t * ldq + (size_t)head * hd;
+    else {
+        const int pos = positions[t];
+        const int page = block_table[(size_t)token_seq[t] * max_blocks + pos / bs];
+        dst = k_pages + (((size_t)page * nkv + (head - nh)) * bs + pos % bs) * hd;
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ss += xv[i] * xv[i];
+    ss = wave_sum(ss);
+    const float scale = 1.0f / sqrtf(ss / (float)hd + eps);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int c = lane + i * 64;
+        if (c < hd) from_float(dst + c, xv[i] * scale * wv[i]);
+    }
+}
+
+FX_API int fx_head_norm_kv_write(void* stream, int dtype, const float* qk, long ldqk, void* q_out, long ldq, const void* v, int ldv,
+                                 const void* wq, const void* wk, int w_dtype, float eps, const int* positions,
+                                 const int* token_seq, const int* block_table, int max_blocks, void* k_pages, void* v_pages,
+                                 int T, int nh, int nkv, int hd, int bs, int vd) {
+    if (vd <= 0) vd = hd;
+    FX_REQUIRE(T >= 0 && nh > 0 && nkv > 0 && bs > 0, "head_norm_kv_write: bad sizes");
+    FX_REQUIRE(hd > 0 && hd <= 256, "head_norm_kv_write: head size %d is outside 1..256", hd);
+    FX_REQUIRE(w_dtype == FX_F32 || w_dtype == FX_BF16, "head_norm_kv_write: unknown weight dtype %d", w_dtype);
+    FX_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "head_norm_kv_write: key and value pages must come together");
+    FX_REQUIRE(!v_pages || v, "head_norm_kv_write: value pages without values");
+    if (T == 0) return 0;
+    const long heads = nh + (k_pages ? nkv : 0);
+    const long norm_blocks = (T * heads + 3) / 4, n_blocks = norm_blocks + (v_pages ? (long)((T + 7) / 8) * nkv : 0);
+    FX_REQUIRE(n_blocks < (1L << 31), "head_norm_kv_write: too many tokens and heads for one launch");
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == FX_F32)
+        head_norm_kv_write_kernel<float><<<(unsigned)n_blocks, 256, 0, s>>>(qk, ldqk, (float*)q_out, ldq, (const float*)v, ldv, wq, wk,
+            w_dtype, eps, positions, token_seq, block_table, max_blocks, (float*)k_pages, (float*)v_pages, T, nh, nkv, hd, bs, vd, (int)norm_blocks);
+    else if (dtype == FX_BF16)
+        head_norm_kv_write_kernel<bf16><<<(unsigned)n_blocks, 256, 0, s>>>(qk, ldqk, (bf16*)q_out, ldq, (const bf16*)v, ldv, wq, wk,
+            w_dtype, eps, positions, token_seq, block_table, max_blocks, (bf16*)k_pages, (bf16*)v_pages, T, nh, nkv, hd, bs, vd, (int)norm_blocks);
+    else
+        return fx_fail("head_norm_kv_write: unknown dtype %d", dtype);
+    FX_CHECK_LAUNCH("head_norm_kv_write");
     return 0;
 }
 

@@ -78,6 +78,9 @@ _sigs = {
                                           c_void_p, c_long, c_void_p, c_void_p, c_long, c_int, c_int, c_int],
     ("recurrent", "fx_gated_head_norm"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int, c_void_p,
                                           c_long, c_int, c_int, c_int, c_float],
+    ("elementwise", "fx_head_norm_kv_write"): [c_void_p, c_int, c_void_p, c_long, c_void_p, c_long, c_void_p, c_int,
+                                               c_void_p, c_void_p, c_int, c_float, c_void_p, c_void_p, c_void_p, c_int,
+                                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int],
     ("elementwise", "fx_residual_add"): [c_void_p, c_int, c_void_p, c_void_p, c_long],
     ("elementwise", "fx_cast"): [c_void_p, c_int, c_void_p, c_int, c_void_p, c_long],
     ("elementwise", "fx_moe_combine"): [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -224,6 +227,44 @@ def rope_kv_write(q, k, v, positions, token_seq, block_table, k_pages, v_pages, 
           _p(_i32(block_table, "block_table")), block_table.shape[1] if block_table is not None else 0,
           _p(k_pages), _p(v_pages), T, n_heads, n_kv_heads, head_dim, block_size, rotary_dim,
           1 if interleaved else 0, _p(rotary_frequencies(q.device, rotary_dim, theta, frequencies)), _p(freq_factors), v_dim)
+
+
+def head_norm_kv_write(qk, q_out, v, q_weight, k_weight, eps, positions, token_seq, block_table, k_pages, v_pages,
+                       n_heads, n_kv_heads, head_dim, block_size, v_dim=None) -> None:
+    """For mixers that norm their heads and rotate nothing, in one launch: every head of the float32 q/k product
+    `qk` [T, (n_heads + n_kv_heads) * head_dim] (or [T, n_heads * head_dim]: no keys) is divided by its root mean
+    square (eps inside the root) and multiplied by `q_weight` / `k_weight` (head_dim elements each, or None); q goes
+    to `q_out` [T, n_heads * head_dim], k into its page, `v` [T, n_kv_heads * v_dim] into its transposed page
+    (`k_pages` None: q alone).  The norms are the bits of `rmsnorm` over gathered heads."""
+    T = qk.shape[0]
+    v_dim = int(v_dim or head_dim)
+    with_keys = k_pages is not None
+    if qk.dtype != torch.float32 or qk.stride(-1) != 1 or qk.shape[1] < (n_heads + (n_kv_heads if with_keys else 0)) * head_dim:
+        raise KernelError(f"head_norm_kv_write: the q/k product must be float32 rows of all heads, got {tuple(qk.shape)} {qk.dtype}")
+    if q_out.stride(-1) != 1 or q_out.shape[0] < T or q_out.shape[1] < n_heads * head_dim:
+        raise KernelError(f"head_norm_kv_write: q_out {tuple(q_out.shape)} for {T} tokens of {n_heads} heads of {head_dim}")
+    w_dtype = FX_F32
+    for w in (q_weight, k_weight):
+        if w is not None:
+            if w.numel() != head_dim or not w.is_contiguous():
+                raise KernelError(f"head_norm_kv_write: a weight of {w.numel()} elements for heads of {head_dim}")
+            w_dtype = dtype_code(w.dtype)
+    if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
+        raise KernelError("head_norm_kv_write: the two weights differ in dtype")
+    if with_keys:
+        if v is None or v.dtype != q_out.dtype or v.stride(-1) != 1 or v.shape[0] < T or v.shape[1] < n_kv_heads * v_dim:
+            raise KernelError("head_norm_kv_write: values must come with the pages, in the type of q_out")
+        if k_pages.dtype != q_out.dtype or v_pages.dtype != q_out.dtype:
+            raise KernelError("cache pages and activations differ in dtype")
+        if tuple(k_pages.shape[1:]) != (n_kv_heads, block_size, head_dim) or \
+                tuple(v_pages.shape[1:]) != (n_kv_heads, v_dim, block_size):
+            raise KernelError(f"cache pages have shapes {tuple(k_pages.shape)}, {tuple(v_pages.shape)}; expected "
+                              f"[pages,{n_kv_heads},{block_size},{head_dim}] and [pages,{n_kv_heads},{v_dim},{block_size}]")
+    _call("elementwise", "fx_head_norm_kv_write", _stream(), dtype_code(q_out.dtype), _p(qk), qk.stride(0), _p(q_out),
+          q_out.stride(0), _p(v) if with_keys else None, v.stride(0) if with_keys else 0, _p(q_weight), _p(k_weight), w_dtype,
+          float(eps), _p(_i32(positions, "positions")), _p(_i32(token_seq, "token_seq")),
+          _p(_i32(block_table, "block_table")), block_table.shape[1] if block_table is not None else 0,
+          _p(k_pages), _p(v_pages) if with_keys else None, T, n_heads, n_kv_heads, head_dim, block_size, v_dim)
 
 
 def residual_add(h: torch.Tensor, y: torch.Tensor) -> None:

@@ -20,6 +20,7 @@ from .base import MIXERS, NORMS, POSITION_ENCODINGS, Mixer, ParamSpec, PartSpec,
 from .linear import Linear, matmul, same_dtype
 
 NO_ROTATION = Rotary(0, 1.0)
+FUSE_HEAD_NORMS = True      # (a switch for tests: the norms of q's and k's heads and the cache write as one launch)
 EVEN_BLOCKS_PER_CU = 250 / 256     # items of 128 queries pay from about one evenly loaded block per CU on (measured on 256 CUs)
 
 
@@ -242,6 +243,22 @@ class PagedAttention(Mixer):
         k = self.k_norm.forward(heads, ctx, rows=k_rows).view(T, self.kvw) if nkv else None
         return q, k, v
 
+    def normed_heads_and_cache(self, x, ctx, units, table, cache):
+        """As `normed_heads` for norms of the RMS form and no rotation, with the cache written by the same launch:
+        returns q [T, qw] and the rest of the product (v, the output gate's rows)."""
+        w, b = self.qkv.weight, self.qkv.bias
+        cut = self.qw + self.kvw
+        qk = matmul(x, w[:cut], bias=None if b is None else b[:cut], epilogue=ops.EPI_STORE_F32)
+        rest = matmul(x, w[cut:], bias=None if b is None else b[cut:]) if w.shape[0] > cut else None
+        q = torch.empty((ctx.n_tokens, self.qw), dtype=ctx.act_dtype, device=qk.device)
+        writes = self.own_kv and cache.writes
+        debug.region("rope + cache write")
+        ops.head_norm_kv_write(qk, q, rest[:, :self.vw] if writes else None, units[0][0], units[1][0], units[0][1],
+                               ctx.positions, ctx.token_seq, table, cache.pages["k"] if writes else None,
+                               cache.pages["v"] if writes else None, self.n_heads, self.n_kv_heads, self.head_dim,
+                               cache.block_size, self.v_dim)
+        return q, rest
+
     def forward(self, x, ctx, cache, residual, qkv=None, post_norm=None) -> None:
         table = ctx.block_tables[cache.group]
         k_pages, v_pages = cache.pages["k"], cache.pages["v"]
@@ -259,8 +276,16 @@ class PagedAttention(Mixer):
             q = qkv[:, :self.qw]
         else:
             gate = None
+            wrote = False
             if self.q_norm is not None:           # every head of q and k through its norm, between bias and rotation
-                q, k, rest = self.normed_heads(x, ctx)
+                units = (self.q_norm.unit_params(), self.k_norm.unit_params())
+                if FUSE_HEAD_NORMS and rot is not None and rot.rotary_dim == 0 and None not in units \
+                        and units[0][1] == units[1][1] and self.head_dim <= 256:
+                    # RMS norms and no rotation: one launch norms the heads and writes q, k's and v's pages
+                    q, rest = self.normed_heads_and_cache(x, ctx, units, table, cache)
+                    k, wrote = None, True
+                else:
+                    q, k, rest = self.normed_heads(x, ctx)
                 qkv = q
                 v = rest[:, :self.vw] if rest is not None else None
                 if self.out_gate:
@@ -276,7 +301,7 @@ class PagedAttention(Mixer):
                 if self.out_gate:
                     gate = qkv[:, cut + self.vw:]
             debug.region("rope + cache write")
-            if self.own_kv:       # (a mixer without keys of its own has no rotation either: nothing to do for its q)
+            if self.own_kv and not wrote:       # (a mixer without keys of its own has no rotation either: nothing to do for its q)
                 if rot is None:
                     self.position.apply(q, k, ctx)
                     rot = NO_ROTATION

@@ -223,6 +223,11 @@ class Norm(Part):
         then call `forward`)."""
         return None
 
+    def unit_params(self):
+        """(weight or None, eps) if this norm is y = x * rsqrt(mean(x^2) + eps) (* weight): what `rms_params` gives,
+        and also a norm of that form without a weight; None for any other norm."""
+        return self.rms_params()
+
 
 @dataclass(frozen=True)
 class Rotary:

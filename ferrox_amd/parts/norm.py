@@ -45,5 +45,8 @@ class RMSNorm(Norm):
         """(weight, eps) of a norm that other parts' kernels may apply themselves; a norm without a weight declines."""
         return (self.weight, self.eps) if self.has_weight else None
 
+    def unit_params(self):
+        return self.weight, self.eps
+
     def forward(self, h, ctx, rows=None):
         return ops.rmsnorm(h, self.weight, self.eps, ctx.act_dtype, rows=rows)

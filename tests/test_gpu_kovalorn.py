@@ -288,6 +288,23 @@ def test_unequal_batches_with_pages_and_slots_used_again(tmp_path_factory, dtype
         assert float(u.row_errors(got_mixed[r], got_alone[r]).max()) <= 2 * u.LIMIT[dtype], r
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_fused_head_norms_give_the_bits_of_the_separate_kernels(tmp_path_factory, dtype, monkeypatch):
+    """The launch that norms the heads of q and k and writes the cache against the three launches it stands for
+    (two norms over gathered heads, the cache write): the same logits bit for bit, prompts, portions and single
+    tokens, also for the layers that have no keys of their own."""
+    from ferrox_amd.parts import attention
+    weights, model = model_for(tmp_path_factory, "main", u.CFG_MAIN, 3, dtype)
+    reqs = {"a": u.random_tokens(u.CFG_MAIN["vocab"], 70, 1), "b": u.random_tokens(u.CFG_MAIN["vocab"], 9, 2)}
+    sched = [[("a", 40), ("b", 2)], [("a", 1), ("b", 7)]] + [[("a", 1)]] * 12 + [[("a", 17)]]
+    got = {}
+    for fused in (True, False):
+        monkeypatch.setattr(attention, "FUSE_HEAD_NORMS", fused)
+        got[fused], _ = u.run_schedule(runner_of(model), reqs, sched)
+    for r in reqs:
+        assert torch.equal(got[True][r], got[False][r]), r
+
+
 def test_used_pages_start_clean_and_passed_pages_come_back(tmp_path_factory):
     """One slot and four pages of 16: every request takes the pages that the one before left.  A layer that keeps
     the first 3 keys and a window of 20 holds a 150-token request in four pages (the first, and up to three under
