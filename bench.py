@@ -462,8 +462,10 @@ def compare_designs(args) -> int:
     sizes = [args.design_size] if args.design_size else sorted(DESIGN_SIZES)
     for size in sizes:
         s = DESIGN_SIZES[size]
-        for name, cfg in design_configs(s).items():
-            if args.design and args.design not in name:
+        configs = design_configs(s)
+        for name, cfg in configs.items():
+            # (a design's whole name means that design alone, any other text every design that holds it)
+            if args.design and args.design != name and (args.design in configs or args.design not in name):
                 continue
             model = random_model(cfg, seed=0, dtype=args.dtype, device="cuda:0")
             bs, T, B = args.block_size, args.ctx, args.batch
