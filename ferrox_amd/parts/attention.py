@@ -178,6 +178,8 @@ class PagedAttention(Mixer):
         """Few tokens: the norm is applied inside the q/k/v product (up to 16 rows it saves a launch; with
         more, every block's reading and norming of all rows costs more than the norm kernel)."""
         rms = norm.rms_params()
+        # (heads that are normed again take their q and k from a float32 product; the norm inside two products, one
+        # of them stored in float32, was measured and is behind the norm kernel: every block norms all rows)
         if (ctx.act_dtype != torch.bfloat16 or rms is None or residual.shape[0] > 16 or self.q_norm is not None
                 or not self.own_kv or not ops.can_fuse_norm(residual, self.qkv.weight, residual.shape[0])):
             return False
@@ -243,13 +245,23 @@ class PagedAttention(Mixer):
         k = self.k_norm.forward(heads, ctx, rows=k_rows).view(T, self.kvw) if nkv else None
         return q, k, v
 
-    def normed_heads_and_cache(self, x, ctx, units, table, cache):
+    def fuses_head_norms(self) -> bool:
+        """Whether the heads' norms and the cache write are one launch: both norms of the RMS form (with or without
+        a weight) under one eps, nothing rotated, no biases."""
+        if not FUSE_HEAD_NORMS or self.q_norm is None or self.bias or self.head_dim > 256:
+            return False
+        rot = self.position.rotary()
+        units = (self.q_norm.unit_params(), self.k_norm.unit_params())
+        return rot is not None and rot.rotary_dim == 0 and None not in units and units[0][1] == units[1][1]
+
+    def normed_heads_and_cache(self, x, ctx, table, cache):
         """As `normed_heads` for norms of the RMS form and no rotation, with the cache written by the same launch:
         returns q [T, qw] and the rest of the product (v, the output gate's rows)."""
-        w, b = self.qkv.weight, self.qkv.bias
+        units = (self.q_norm.unit_params(), self.k_norm.unit_params())
+        w = self.qkv.weight
         cut = self.qw + self.kvw
-        qk = matmul(x, w[:cut], bias=None if b is None else b[:cut], epilogue=ops.EPI_STORE_F32)
-        rest = matmul(x, w[cut:], bias=None if b is None else b[cut:]) if w.shape[0] > cut else None
+        qk = matmul(x, w[:cut], epilogue=ops.EPI_STORE_F32)
+        rest = matmul(x, w[cut:]) if w.shape[0] > cut else None
         q = torch.empty((ctx.n_tokens, self.qw), dtype=ctx.act_dtype, device=qk.device)
         writes = self.own_kv and cache.writes
         debug.region("rope + cache write")
@@ -278,11 +290,9 @@ class PagedAttention(Mixer):
             gate = None
             wrote = False
             if self.q_norm is not None:           # every head of q and k through its norm, between bias and rotation
-                units = (self.q_norm.unit_params(), self.k_norm.unit_params())
-                if FUSE_HEAD_NORMS and rot is not None and rot.rotary_dim == 0 and None not in units \
-                        and units[0][1] == units[1][1] and self.head_dim <= 256:
+                if self.fuses_head_norms():
                     # RMS norms and no rotation: one launch norms the heads and writes q, k's and v's pages
-                    q, rest = self.normed_heads_and_cache(x, ctx, units, table, cache)
+                    q, rest = self.normed_heads_and_cache(x, ctx, table, cache)
                     k, wrote = None, True
                 else:
                     q, k, rest = self.normed_heads(x, ctx)
