@@ -353,6 +353,31 @@ def test_keys_at_the_edges_stand_out(tmp_path_factory, dtype):
         run_and_check(cfg, weights, model, reqs, sched, dtype, f"edge {first}")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_far_key_among_hundreds(tmp_path_factory, dtype):
+    """A layer without a mask under a peaked softmax: queries deep in a 600-token sequence pick keys hundreds of
+    positions back (the plain model without the keys beyond 400 positions differs far beyond the limit), across
+    nine pages of 64, whole, in portions, and decoded one by one; a second layer reads the same keys under a window."""
+    scale, bar = {"float32": (2.0, 0.15), "bfloat16": (0.8, 0.09)}[dtype]
+    cfg = u.config([u.attention_layer(heads=4, kv_heads=2, dim=32, vdim=32, window=0, scale=scale, mlp=u.dense(64)),
+                    u.attention_layer(heads=2, kv_heads=2, dim=32, vdim=32, window=70, keep_first=0, scale=scale, kv_from=0)], width=64)
+
+    def no_sink(w):
+        for i in range(2):
+            w[f"l{i}.mix.sink"] = w[f"l{i}.mix.sink"] - 6.0
+
+    weights, model = model_for(tmp_path_factory, "far" + dtype, cfg, 23, dtype, change=no_sink)
+    tokens = u.random_tokens(cfg["vocab"], 600, 6)
+    near = dict(cfg, layers=[dict(cfg["layers"][0], mixer=dict(cfg["layers"][0]["mixer"], mask={"size": 400, "keep_first": 0})),
+                             cfg["layers"][1]])
+    moved = u.row_errors(plain.forward(near, weights, tokens)[400:], plain.forward(cfg, weights, tokens)[400:])
+    assert float(moved.max()) > bar, float(moved.max())
+    reqs = {"f": tokens}
+    for what, sched in (("whole", [[("f", 600)]]), ("decode", [[("f", 560)]] + [[("f", 1)]] * 40),
+                        ("portions", [[("f", 37)]] * 16 + [[("f", 8)]])):
+        run_and_check(cfg, weights, model, reqs, sched, dtype, "far " + what, block_size=64, num_pages=10)
+
+
 def test_a_sink_that_takes_nearly_all(tmp_path_factory):
     """Sinks far above every score (the heads' outputs nearly vanish) and far below (no sink at all): neither
     overflows, both match the plain model."""
